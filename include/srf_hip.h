@@ -231,8 +231,12 @@ typedef struct srf_render_args {
 	int32_t  network_output_dtype;
 } srf_render_args;
 
-/* Waits for `stream` and reports whether the ordered-offset chain of the last training compositing call completed.
- * No counterpart in the reference (its offsets come from one atomicAdd per ray and cannot fail this way). */
+/* Waits for `stream` and reports whether the ordered-offset chain of the training compositing calls so far completed.
+ * No counterpart in the reference (its offsets come from one atomicAdd per ray and cannot fail this way).
+ * The streaming kernel's workgroups wait, with a bound, for the sample counts of the groups before theirs.  If a wait runs
+ * out, that call's compacted counter reads 0xffffffff, every ray of the affected groups gets a zero count and no gradients, and
+ * the failure is returned by this function or by the next srf_marcher_volume_rendering_with_loss_and_gradient on the marcher,
+ * whichever comes first; from then on the marcher uses the three-launch implementation, which has no such waits. */
 int  srf_marcher_sync_check(srf_marcher_t* m, void* stream);
 
 /* RayMarcher::volume_rendering, ray_marcher.cu:376-415 (kernel :204-282) */
@@ -240,8 +244,9 @@ int  srf_marcher_volume_rendering(srf_marcher_t* m, const srf_sampler_t* s, cons
                                   srf_ray_payload* payloads, float* rgba, const float* coords, const void* rgbsigma, void* stream);
 
 /* ---------------- orchestrator kernels ---------------- */
-/* compact_rays_kernel, internal/testbed.cu:423-446; survivors keep their relative order. Counters are device uint32, caller-zeroed. */
-int  srf_compact_rays(uint32_t n_elements, const srf_ray_payload* src_payloads, const float* src_rgba,
+/* compact_rays_kernel, internal/testbed.cu:423-446; survivors keep their relative order. Counters are device uint32, caller-zeroed.
+ * The marcher owns the scratch the ordered compaction needs (flags and positions, 16 bytes per ray). */
+int  srf_compact_rays(srf_marcher_t* m, uint32_t n_elements, const srf_ray_payload* src_payloads, const float* src_rgba,
                       srf_ray_payload* dst_payloads, float* dst_rgba, srf_ray_payload* final_payloads, float* final_rgba,
                       uint32_t* n_alive_counter, uint32_t* n_final_counter, void* stream);
 /* shade_kernel, internal/testbed.cu:448-477 */
@@ -267,7 +272,10 @@ int  srf_render_frame_fused(srf_sampler_t* s, const srf_marcher_t* m, const srf_
 int  srf_field_eval(const srf_sampler_t* s, const srf_field* field, uint32_t n_coords, const float* coords,
                     void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream);
 
-/* ---------------- test hook ---------------- */
+/* ---------------- test hooks ---------------- */
+/* number of polls a workgroup of the streaming compositing kernel makes before it gives up waiting for its predecessors
+ * (default 2^22).  0 lets a test exercise the give-up path without any kernel waiting for long. */
+int  srf_marcher_debug_set_lookback_spin_limit(srf_marcher_t* m, uint32_t polls);
 /* evaluates one of the shared elementary functions on the device over n inputs:
  * which = 0 exp, 1 log, 2 sin, 3 cos, 4 asin, 5 atan2(a,b), 6 pow(a,b), 7 sqrt, 8 a/b, 9 float->half->float,
  * 10 1/a (the reciprocal of the disparity stepping) */

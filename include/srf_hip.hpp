@@ -166,9 +166,9 @@ private:
 };
 
 // Testbed's helper launches (testbed.cu:398-404, 423-477)
-inline void compact_rays(uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba, srf_ray_payload* dst_payloads, float* dst_rgba,
+inline void compact_rays(const RayMarcher& marcher, uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba, srf_ray_payload* dst_payloads, float* dst_rgba,
                          srf_ray_payload* final_payloads, float* final_rgba, uint32_t* n_alive_counter, uint32_t* n_final_counter, void* stream) {
-	check(srf_compact_rays(n, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba, n_alive_counter, n_final_counter, stream));
+	check(srf_compact_rays(marcher.handle(), n, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba, n_alive_counter, n_final_counter, stream));
 }
 inline void shade(uint32_t n_rays, const float* rgba, const srf_ray_payload* payloads, float* frame_buffer, int32_t render_mode, bool train_in_linear_colors, void* stream) {
 	check(srf_shade(n_rays, rgba, payloads, frame_buffer, render_mode, train_in_linear_colors ? 1 : 0, stream));

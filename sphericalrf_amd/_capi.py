@@ -95,7 +95,7 @@ SYMBOLS = [
     "srf_marcher_config_default", "srf_marcher_create", "srf_marcher_destroy", "srf_marcher_get_config", "srf_marcher_set_config",
     "srf_marcher_volume_rendering_with_loss_and_gradient", "srf_marcher_sync_check", "srf_marcher_volume_rendering",
     "srf_compact_rays", "srf_shade", "srf_fill_rollover", "srf_fill_rollover_and_rescale",
-    "srf_render_frame_fused", "srf_field_eval", "srf_debug_eval_elem",
+    "srf_render_frame_fused", "srf_field_eval", "srf_debug_eval_elem", "srf_marcher_debug_set_lookback_spin_limit",
 ]
 
 
@@ -147,7 +147,8 @@ def load():
     L.srf_marcher_volume_rendering_with_loss_and_gradient.argtypes = [vp, P(LossArgs), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     L.srf_marcher_sync_check.argtypes = [vp, vp]
     L.srf_marcher_volume_rendering.argtypes = [vp, vp, P(RenderArgs), vp, vp, vp, vp, vp]
-    L.srf_compact_rays.argtypes = [u32, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    L.srf_compact_rays.argtypes = [vp, u32, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    L.srf_marcher_debug_set_lookback_spin_limit.argtypes = [vp, u32]
     L.srf_shade.argtypes = [u32, vp, vp, vp, i32, i32, vp]
     L.srf_fill_rollover.argtypes = [u32, u32, vp, vp, vp]
     L.srf_fill_rollover_and_rescale.argtypes = [u32, u32, vp, vp, i32, vp]

@@ -148,36 +148,43 @@ class Dataset:
         return d
 
 
+def sampler_config_from_dict(config):
+    """the "samlper" JSON block (a dict) as srf_sampler_config: the reference's keys and defaults, occupancy_sampler.cu:911-943"""
+    L = K.load()
+    cfg = K.SamplerConfig()
+    L.srf_sampler_config_default(C.byref(cfg))
+    cfg.warping_type = string_to_warping_type(config.get("warping_type", "NGP"))
+    cfg.aabb_scale = float(config.get("aabb_scale", 1))
+    cfg.use_grid = int(bool(config.get("use_grid", True)))
+    cfg.init_grid_with_mask = int(bool(config.get("init_grid_with_mask", True)))
+    gs = config.get("grid_size", 128)
+    gs = (gs, gs, gs) if isinstance(gs, int) else tuple(gs)
+    cfg.grid_size = (K.u32 * 3)(*gs)
+    cfg.num_cascades = int(config.get("num_cascades", 1))
+    cfg.ema_decay = float(config.get("ema_decay", 0.95))
+    if cfg.use_grid:
+        # the reference parses this key only when use_grid is set, and its default "Exp" is not a valid name
+        cfg.grid_distribution_type = string_to_griddist_type(config.get("grid_distribution_type", "Exp"))
+    cfg.maximum_marching_steps = int(config.get("maximum_marching_steps", 1024))
+    cfg.cone_angle_constant = float(config.get("cone_angle_constant", 0.0))
+    cfg.min_cone_stepsize = float(config.get("min_cone_stepsize", -1.0))
+    cfg.max_cone_stepsize = float(config.get("max_cone_stepsize", -1.0))
+    cfg.near_distance = float(config.get("near_distance", 0.2))
+    cfg.far_distance = float(config.get("far_distance", 100.0))
+    cfg.sampling_type = string_to_sampling_type(config.get("sampling_type", "Original"))
+    cfg.snap_to_pixel_centers_in_training = int(bool(config.get("snap_to_pixel_centers_in_training", True)))
+    cfg.snap_to_pixel_centers_in_rendering = int(bool(config.get("snap_to_pixel_centers_in_rendering", True)))
+    cfg.min_optical_thickness = float(config.get("min_optical_thickness", 0.01))
+    return cfg
+
+
 class OccupancySampler:
     """internal/sampler/occupancy_sampler.h:13-135.  `config` is the "samlper" JSON block as a dict."""
 
     def __init__(self, config):
         self._h = None
         L = K.load()
-        cfg = K.SamplerConfig()
-        L.srf_sampler_config_default(C.byref(cfg))
-        cfg.warping_type = string_to_warping_type(config.get("warping_type", "NGP"))
-        cfg.aabb_scale = float(config.get("aabb_scale", 1))
-        cfg.use_grid = int(bool(config.get("use_grid", True)))
-        cfg.init_grid_with_mask = int(bool(config.get("init_grid_with_mask", True)))
-        gs = config.get("grid_size", 128)
-        gs = (gs, gs, gs) if isinstance(gs, int) else tuple(gs)
-        cfg.grid_size = (K.u32 * 3)(*gs)
-        cfg.num_cascades = int(config.get("num_cascades", 1))
-        cfg.ema_decay = float(config.get("ema_decay", 0.95))
-        if cfg.use_grid:
-            # the reference parses this key only when use_grid is set, and its default "Exp" is not a valid name
-            cfg.grid_distribution_type = string_to_griddist_type(config.get("grid_distribution_type", "Exp"))
-        cfg.maximum_marching_steps = int(config.get("maximum_marching_steps", 1024))
-        cfg.cone_angle_constant = float(config.get("cone_angle_constant", 0.0))
-        cfg.min_cone_stepsize = float(config.get("min_cone_stepsize", -1.0))
-        cfg.max_cone_stepsize = float(config.get("max_cone_stepsize", -1.0))
-        cfg.near_distance = float(config.get("near_distance", 0.2))
-        cfg.far_distance = float(config.get("far_distance", 100.0))
-        cfg.sampling_type = string_to_sampling_type(config.get("sampling_type", "Original"))
-        cfg.snap_to_pixel_centers_in_training = int(bool(config.get("snap_to_pixel_centers_in_training", True)))
-        cfg.snap_to_pixel_centers_in_rendering = int(bool(config.get("snap_to_pixel_centers_in_rendering", True)))
-        cfg.min_optical_thickness = float(config.get("min_optical_thickness", 0.01))
+        cfg = sampler_config_from_dict(config)
         h = C.c_void_p()
         K.check(L.srf_sampler_create(C.byref(cfg), C.byref(h)))
         self._h = h
@@ -376,8 +383,12 @@ class RayMarcher:
             _dev(rgb_ray_out, torch.float32, 3 * n_rays, "rgb_ray_out", allow_none=True), _stream()))
 
     def sync_check(self):
-        """wait for the current stream and raise if the last training compositing call could not order its offsets"""
+        """wait for the current stream and raise if a training compositing call could not order its offsets"""
         K.check(self._L.srf_marcher_sync_check(self._h, _stream()))
+
+    def debug_set_lookback_spin_limit(self, polls):
+        """test hook: polls a workgroup of the streaming kernel makes before it gives up waiting for its predecessors"""
+        K.check(self._L.srf_marcher_debug_set_lookback_spin_limit(self._h, int(polls)))
 
     def volume_rendering(self, sampler, n_rays, n_steps, i_steps_offset, payloads, rgba, coords, rgbsigma, padded_output_width=4,
                          density_activation=K.ACT_EXPONENTIAL, rgb_activation=K.ACT_LOGISTIC, render_mode=K.RENDER_SHADE,
@@ -394,8 +405,9 @@ class RayMarcher:
 
 
 # ---- orchestrator kernels (internal/testbed.cu:398-404, 423-477) ---------------------------------
-def compact_rays(n_elements, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba, n_alive_counter, n_final_counter):
-    K.check(K.load().srf_compact_rays(n_elements, _dev(src_payloads, torch.uint8, 40 * n_elements), _dev(src_rgba, torch.float32, 4 * n_elements),
+def compact_rays(marcher, n_elements, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba, n_alive_counter, n_final_counter):
+    """compact_rays_kernel (internal/testbed.cu:423-446); `marcher` (a RayMarcher) owns the scratch of the ordered compaction"""
+    K.check(K.load().srf_compact_rays(marcher._h, n_elements, _dev(src_payloads, torch.uint8, 40 * n_elements), _dev(src_rgba, torch.float32, 4 * n_elements),
                                       _dev(dst_payloads, torch.uint8, 40 * n_elements), _dev(dst_rgba, torch.float32, 4 * n_elements),
                                       _dev(final_payloads, torch.uint8, 40 * n_elements), _dev(final_rgba, torch.float32, 4 * n_elements),
                                       _dev(n_alive_counter, torch.int32, 1), _dev(n_final_counter, torch.int32, 1), _stream()))

@@ -52,5 +52,18 @@ def build(verbose=False, extra_flags=()):
     return LIB
 
 
+def build_step_bench():
+    """The native harness tests/cpp/step_bench (C++ over include/srf_hip.hpp; no Python at run time)."""
+    root = os.path.dirname(_HERE)
+    src = os.path.join(root, "tests", "cpp", "step_bench.cpp")
+    exe = os.path.join(root, "tests", "cpp", "step_bench")
+    cmd = [hipcc(), "--offload-arch=gfx950", "-O2", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I", os.path.join(root, "include"), src, "-L", LIBDIR, "-lsrf_hip", "-Wl,-rpath,$ORIGIN/../../sphericalrf_amd/lib", "-o", exe]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("step_bench build failed:\n%s" % r.stdout)
+    return exe
+
+
 if __name__ == "__main__":
     print(build(verbose=True, extra_flags=sys.argv[1:]))

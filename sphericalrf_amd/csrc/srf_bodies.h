@@ -871,6 +871,8 @@ struct LossConst {
 	float    min_optical_thickness;
 	int32_t  use_grid;
 	float    bg_in[3];                 // background before srgb_to_linear (the shared random draw already applied)
+	float    bg_lin[3];                // srgb_to_linear(bg_in): the same for every ray of a call, so worked out once (loss_const_background)
+	float    bg_enc[3];                // linear_to_srgb(bg_lin)
 	int32_t  color_space;
 	int32_t  train_in_linear;
 	float    thr;
@@ -884,17 +886,22 @@ struct FwdRay {
 	uint32_t numsteps, base;
 };
 
+// ray_marcher.cu:85-86, :94, :100 — the two encodings of the background colour that every ray of a call uses; after bg_in is set
+SRF_HD void loss_const_background(LossConst& K) {
+	for (int c = 0; c < 3; ++c) { K.bg_lin[c] = srgb_to_linear(K.bg_in[c]); K.bg_enc[c] = linear_to_srgb(K.bg_lin[c]); }
+}
+
 // ray_marcher.cu:85-104 — background and ground-truth colour of a ray
 SRF_HD void target_and_background(const LossConst& K, Float4 tex, float target[3], float bg[3]) {
-	for (int c = 0; c < 3; ++c) { bg[c] = srgb_to_linear(K.bg_in[c]); target[c] = 0.f; }
+	for (int c = 0; c < 3; ++c) { bg[c] = K.bg_lin[c]; target[c] = 0.f; }
 	if (K.train_in_linear || K.color_space == SRF_COLOR_LINEAR) {
 		const float k = 1 - tex.w;
 		target[0] = tex.x + k * bg[0]; target[1] = tex.y + k * bg[1]; target[2] = tex.z + k * bg[2];
 		if (!K.train_in_linear) {
-			for (int c = 0; c < 3; ++c) { target[c] = linear_to_srgb(target[c]); bg[c] = linear_to_srgb(bg[c]); }
+			for (int c = 0; c < 3; ++c) { target[c] = linear_to_srgb(target[c]); bg[c] = K.bg_enc[c]; }
 		}
 	} else if (K.color_space == SRF_COLOR_SRGB) {
-		for (int c = 0; c < 3; ++c) bg[c] = linear_to_srgb(bg[c]);
+		for (int c = 0; c < 3; ++c) bg[c] = K.bg_enc[c];
 		if (tex.w > 0) {
 			const float k = 1 - tex.w;
 			target[0] = linear_to_srgb(tex.x / tex.w) * tex.w + k * bg[0];

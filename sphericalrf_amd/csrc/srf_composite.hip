@@ -40,51 +40,75 @@ __global__ void __launch_bounds__(128) k_volume_rendering(Params P, srf_render_a
 // ------------------------------------------------------------------------------------
 // Single-launch compositing (phases in srf_composite_fused.h)
 // ------------------------------------------------------------------------------------
-// Ordered offsets across workgroups.  Every group publishes the number of samples it keeps; a
-// group's offset is the sum over all groups before it.  Groups are bundled into segments of 64:
-// inside a segment a group adds up its predecessors' counts with one 64-wide read; the last
-// group of a segment also publishes the segment's total, and the sum over earlier segments is
-// found by a decoupled look-back over segment entries (flag 1 = total of that segment alone,
-// flag 2 = total of everything up to and including it).  With a few thousand groups in flight
-// both steps usually finish in one or two memory round trips, where a single-level look-back
-// would have to walk back over every group in flight.
+// Ordered offsets across items (an item: the rays of a group that a streaming workgroup takes at a time, see
+// fused::items_of_group).  Every item publishes the number of samples it keeps; an
+// item's offset is the sum over all items before it.  Items are bundled into segments of 64:
+// inside a segment an item adds up its predecessors' counts with one 64-wide read; a
+// segment's total is accumulated as its items publish (complete once all 64 have), and the sum
+// over earlier segments is found by a decoupled look-back over segment entries (the totals of
+// complete segments, back to the nearest segment for which somebody has left the sum of everything
+// up to and including it).  With a few thousand items in flight both steps usually finish in one
+// memory round trip, where a single-level look-back would have to walk back over every item in flight.
+constexpr uint32_t PREPARE_WAVES = 16;   // groups per workgroup of k_chain_prepare
+// Segment totals lie this many 8-byte words apart: every item in flight adds to one of a few neighbouring segments' totals, and
+// additions to one stretch of memory take turns
+constexpr uint32_t SEG_STRIDE = 32;
 struct ChainScratch {
-	unsigned long long* group_status;   // per group:   flag << 32 | count (flag 1)
-	unsigned long long* seg_status;     // per segment: flag << 32 | count (flag 1 total, 2 inclusive prefix)
+	unsigned long long* item_status;    // per item:    flag << 32 | count (flag 1; 3 = gave up)
+	unsigned long long* seg_status;     // per segment of 64 items: items published so far << 32 | sum of their counts
+	unsigned long long* seg_prefix;     // per segment: flag << 32 | count (flag 2: everything up to and including the segment, 3 = an item gave up)
 	uint32_t* initial;                  // value of the compacted counter before the launch
-	uint32_t* error;
-	unsigned long long* timing;   // SRF_FUSED_TIMING builds: cycles per phase summed over groups
+	uint32_t* error;                    // device word: set when an item gave up
+	uint32_t* slow_count;               // number of entries of slow_items
+	uint32_t* n_items;                  // number of items
+	uint32_t* group_words;              // per group: how many items it makes (fused::group_items_word)
+	uint32_t* prepare_sums;             // per workgroup of k_chain_prepare: how many items its groups make
+	U2* items;                          // the items in ray order (fused::items_of_group)
+	uint32_t* slow_items;               // items of groups that the streaming path does not take (see k_chain_prepare)
+	uint32_t* side;                     // per ray of such a group: samples consumed (forward kernel), then compacted offset (streaming kernel)
+	uint32_t* host_error;               // like error, in host memory the device can write (may be NULL)
+	uint32_t spin_limit;                // polls an item makes before it gives up
 };
 
-// Ordering point between the phases of a group.  A group of one wavefront needs no hardware barrier: the
-// wave's LDS operations execute in program order, so only the compiler has to be kept from moving them
-// across; and unlike __syncthreads() this does not wait for the global loads that were requested early
-// on purpose.  Larger groups use the ordinary barrier.
-__device__ __forceinline__ void group_sync() {
-	if (fused::THREADS == WAVE) __builtin_amdgcn_wave_barrier();
-	else __syncthreads();
+// bytes of device scratch the chain needs for n_rays rays, and where its parts lie (a group makes at most two items)
+struct ChainLayout { size_t off_seg, off_prefix, off_misc, off_words, off_sums, off_items, off_list, off_side, bytes; };
+SRF_HD ChainLayout chain_layout(uint32_t n_rays) {
+	const size_t n_groups = ((size_t)n_rays + fused::RAYS - 1) / fused::RAYS;
+	const size_t n_items = 2 * n_groups;
+	ChainLayout L;
+	L.off_seg = (n_items * 8 + 255) / 256 * 256;
+	L.off_prefix = (L.off_seg + (n_items + 63) / 64 * 8 * SEG_STRIDE + 255) / 256 * 256;
+	L.off_misc = (L.off_prefix + (n_items + 63) / 64 * 8 + 255) / 256 * 256;
+	L.off_words = L.off_misc + 512;
+	L.off_sums = (L.off_words + n_groups * 4 + 255) / 256 * 256;
+	L.off_items = (L.off_sums + (n_groups / PREPARE_WAVES + 1) * 4 + 255) / 256 * 256;
+	L.off_list = (L.off_items + n_items * 8 + 255) / 256 * 256;
+	L.off_side = (L.off_list + n_groups * 4 + 255) / 256 * 256;
+	L.bytes = L.off_side + n_groups * fused::RAYS * 4;
+	return L;
+}
+static ChainScratch chain_scratch_at(void* base, uint32_t n_rays, uint32_t* host_error, uint32_t spin_limit) {
+	const ChainLayout L = chain_layout(n_rays);
+	ChainScratch S;
+	S.item_status = (unsigned long long*)base;
+	S.seg_status = (unsigned long long*)((char*)base + L.off_seg);
+	S.seg_prefix = (unsigned long long*)((char*)base + L.off_prefix);
+	S.initial = (uint32_t*)((char*)base + L.off_misc);
+	S.error = S.initial + 1;
+	S.slow_count = S.initial + 2;
+	S.n_items = S.initial + 3;
+	S.group_words = (uint32_t*)((char*)base + L.off_words);
+	S.prepare_sums = (uint32_t*)((char*)base + L.off_sums);
+	S.items = (U2*)((char*)base + L.off_items);
+	S.slow_items = (uint32_t*)((char*)base + L.off_list);
+	S.side = (uint32_t*)((char*)base + L.off_side);
+	S.host_error = host_error;
+	S.spin_limit = spin_limit;
+	return S;
 }
 
-#ifdef SRF_FUSED_TIMING
-#define SRF_TSTAMP(k) do { if (tid == 0) { const unsigned long long now_ = clock64(); t_acc_[k] += now_ - t_prev_; t_prev_ = now_; } } while (0)
-#else
-#define SRF_TSTAMP(k) ((void)0)
-#endif
-
-__global__ void k_fill_word(uint32_t* p, uint32_t v) { *p = v; }
-
-__global__ void k_chain_init(ChainScratch S, uint32_t n_groups, const uint32_t* __restrict__ counter) {
-	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-	if (i < n_groups) S.group_status[i] = 0ull;
-	if (i < (n_groups + 63) / 64) S.seg_status[i] = 0ull;
-	if (i == 0) *S.initial = *counter;
-}
-
-constexpr uint32_t LOOKBACK_SPIN_LIMIT = 1u << 22;
-
-#ifndef SRF_LOOKBACK_SLEEP
-#define SRF_LOOKBACK_SLEEP 2
-#endif
+constexpr uint32_t LOOKBACK_SLEEP = 2;
+constexpr uint32_t CHAIN_FAILED = 0xffffffffu;   // prefix of a group whose look-back gave up; also what the compacted counter reads then
 
 __device__ inline unsigned long long status_load(const unsigned long long* p) {
 	return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -93,410 +117,498 @@ __device__ inline void status_store(unsigned long long* p, uint32_t flag, uint32
 	__hip_atomic_store(p, ((unsigned long long)flag << 32) | value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Exclusive prefix of group g over the groups before it, by the 64 lanes of one wave.  A group only
-// waits for lower-numbered groups.  Both levels are read in the same round trip (each lane loads one
-// group entry of its own segment and one segment entry); a round is repeated until nothing it needs
-// is missing.  Every wait is bounded: past the limit an error flag is raised and the prefix is
-// abandoned, so the grid always drains.
-__device__ inline uint32_t chained_prefix(const ChainScratch& S, uint32_t g, uint32_t total) {
+// An item's count, visible to every item after it (one lane): its own status word, and its share of its segment's running total.
+__device__ inline void chain_publish(const ChainScratch& S, uint32_t i, uint32_t total) {
+	if (lane_id() == 0) {
+		status_store(&S.item_status[i], 1u, total);
+		(void)__hip_atomic_fetch_add(&S.seg_status[(size_t)(i / WAVE) * SEG_STRIDE], (1ull << 32) | total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+	}
+}
+
+// Exclusive prefix of item i over the items before it, by the 64 lanes of one wave.  An item only waits for
+// lower-numbered items.  Both levels are read in the same round trip (each lane loads one item entry of its own
+// segment and the entries of one earlier segment); a round is repeated until nothing it needs is missing.  The first round's
+// loads can be requested long before their values are needed (chain_peek), so that the round trip overlaps other work; the words
+// only ever move from "missing" to "there", so an early value is either final or asks for another round.  Everything an item
+// needs is put there when its predecessors publish their counts, never when they resolve their own prefixes, so an item waits only
+// for a workgroup that has fallen behind by the time that passes between an item's count and its look-back.
+// Every wait is bounded: past the limit, or when a predecessor has given up, the item gives up too: it marks its own
+// entries so that its successors stop at once, raises the error words and returns CHAIN_FAILED.
+struct ChainPeek { unsigned long long vg, vs, vp; uint32_t initial; };
+
+__device__ inline ChainPeek chain_peek(const ChainScratch& S, uint32_t i) {
 	const uint32_t lane = lane_id();
-	const uint32_t seg = g / WAVE, j = g % WAVE;
-	const bool closes_segment = j == WAVE - 1;
-	if (lane == 0) status_store(&S.group_status[g], 1u, total);
-	const uint32_t initial = *S.initial;
+	const uint32_t seg = i / WAVE, j = i % WAVE;
+	ChainPeek p;
+	p.initial = *S.initial;
+	p.vg = 1ull << 32;
+	if (j != 0 && lane < j) p.vg = status_load(&S.item_status[seg * WAVE + lane]);
+	p.vs = 0ull;
+	p.vp = (2ull << 32) | p.initial;                  // before the first segment: the counter's value before the launch
+	const int64_t idx = (int64_t)seg - 1 - (int64_t)lane;
+	if (idx >= 0) { p.vs = status_load(&S.seg_status[(size_t)idx * SEG_STRIDE]); p.vp = status_load(&S.seg_prefix[idx]); }
+	return p;
+}
+
+__device__ inline uint32_t chain_resolve(const ChainScratch& S, uint32_t i, uint32_t total, const ChainPeek& peek) {
+	const uint32_t lane = lane_id();
+	const uint32_t seg = i / WAVE, j = i % WAVE;
+	const uint32_t initial = peek.initial;
 	uint32_t spins = 0, within = 0, before = 0;
-	bool have_within = j == 0, published_total = false;
+	bool have_within = j == 0, have_before = false, failed = false, first = true;
 	int64_t hi = (int64_t)seg - 1;
 	for (;;) {
-		unsigned long long vg = 1ull << 32;
-		if (!have_within && lane < j) vg = status_load(&S.group_status[seg * WAVE + lane]);
-		const int64_t idx = hi - (int64_t)lane;
-		unsigned long long vs = (2ull << 32) | initial;
-		if (idx >= 0) vs = status_load(&S.seg_status[idx]);
-		if (!have_within && __ballot((uint32_t)(vg >> 32) == 0u) == 0ull) {
+		unsigned long long vg = 1ull << 32, vs = 0ull, vp = (2ull << 32) | initial;
+		if (first) {
+			vg = peek.vg; vs = peek.vs; vp = peek.vp;
+		} else {
+			if (!have_within && lane < j) vg = status_load(&S.item_status[seg * WAVE + lane]);
+			const int64_t idx = hi - (int64_t)lane;
+			if (!have_before && idx >= 0) { vs = status_load(&S.seg_status[(size_t)idx * SEG_STRIDE]); vp = status_load(&S.seg_prefix[idx]); }
+		}
+		first = false;
+		const uint32_t gflag = (uint32_t)(vg >> 32), pflag = (uint32_t)(vp >> 32);
+		if (__ballot(gflag == 3u) != 0ull) { failed = true; break; }
+		if (!have_within && __ballot(gflag == 0u) == 0ull) {
 			within = wave_sum_u32(lane < j ? (uint32_t)vg : 0u);
 			have_within = true;
 		}
-		if (have_within && closes_segment && !published_total) {
-			if (lane == 0) status_store(&S.seg_status[seg], 1u, within + total);
-			published_total = true;
+		if (!have_before) {
+			// a segment's entry: its inclusive prefix (left by whoever has resolved past it), else its total once all of its items have published
+			const bool complete = (uint32_t)(vs >> 32) == WAVE;
+			const unsigned long long has_prefix = __ballot(pflag == 2u);
+			const unsigned long long missing = __ballot(pflag != 2u && pflag != 3u && !complete);
+			const unsigned long long poisoned = __ballot(pflag == 3u);
+			const uint32_t first_prefix = has_prefix ? (uint32_t)__builtin_ctzll(has_prefix) : 64u;
+			const uint32_t first_missing = missing ? (uint32_t)__builtin_ctzll(missing) : 64u;
+			const uint32_t first_poisoned = poisoned ? (uint32_t)__builtin_ctzll(poisoned) : 64u;
+			if (first_poisoned < first_prefix && first_poisoned < first_missing) { failed = true; break; }
+			if (first_prefix < first_missing) {
+				before += wave_sum_u32(lane < first_prefix ? (uint32_t)vs : (lane == first_prefix ? (uint32_t)vp : 0u));
+				have_before = true;
+			} else if (first_missing == 64u) { before += wave_sum_u32((uint32_t)vs); hi -= 64; continue; }   // 64 totals, no prefix yet: look further back
 		}
-		const uint32_t flag = (uint32_t)(vs >> 32), val = (uint32_t)vs;
-		const unsigned long long has_prefix = __ballot(flag == 2u);
-		const unsigned long long missing = __ballot(flag == 0u);
-		const uint32_t first_prefix = has_prefix ? (uint32_t)__builtin_ctzll(has_prefix) : 64u;
-		const uint32_t first_missing = missing ? (uint32_t)__builtin_ctzll(missing) : 64u;
-		bool have_before = false;
-		if (first_prefix < first_missing) { before += wave_sum_u32(lane <= first_prefix ? val : 0u); have_before = true; }
-		else if (first_missing == 64u) { before += wave_sum_u32(val); hi -= 64; continue; }   // 64 totals, no prefix yet: look further back
-		if (have_before) {
-			if (have_within) break;
-			// the segment part arrived; only the group entries are still missing: keep the sum, poll them alone
-			for (;;) {
-				const unsigned long long v2 = lane < j ? status_load(&S.group_status[seg * WAVE + lane]) : (1ull << 32);
-				if (__ballot((uint32_t)(v2 >> 32) == 0u) == 0ull) { within = wave_sum_u32(lane < j ? (uint32_t)v2 : 0u); have_within = true; break; }
-				if (++spins > LOOKBACK_SPIN_LIMIT) break;
-				__builtin_amdgcn_s_sleep(SRF_LOOKBACK_SLEEP);
-			}
-			if (have_within && closes_segment && !published_total) {
-				if (lane == 0) status_store(&S.seg_status[seg], 1u, within + total);
-				published_total = true;
-			}
-			break;
+		if (have_before && have_within) break;
+		if (++spins > S.spin_limit) { failed = true; break; }
+		__builtin_amdgcn_s_sleep(LOOKBACK_SLEEP);
+	}
+	if (failed) {
+		if (lane == 0) {
+			status_store(&S.item_status[i], 3u, 0u);
+			status_store(&S.seg_prefix[seg], 3u, 0u);
+			atomicExch(S.error, 1u);
+			if (S.host_error) __hip_atomic_store(S.host_error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 		}
-		if (++spins > LOOKBACK_SPIN_LIMIT) break;
-		__builtin_amdgcn_s_sleep(SRF_LOOKBACK_SLEEP);
+		return CHAIN_FAILED;
 	}
-	if (spins > LOOKBACK_SPIN_LIMIT || !have_within) {
-		if (lane == 0) atomicExch(S.error, 1u);
-		return 0;
+	// shortcuts for later look-backs: the prefix up to the end of the segment before this one, and up to the end of this one
+	if (lane == 0) {
+		if (j == 0 && seg != 0) status_store(&S.seg_prefix[seg - 1], 2u, before);
+		if (j == WAVE - 1) status_store(&S.seg_prefix[seg], 2u, before + within + total);
 	}
-	if (closes_segment && lane == 0) status_store(&S.seg_status[seg], 2u, before + within + total);
 	return before + within;
 }
 
-// Four workgroups per CU: the window of 1792 samples keeps a group's LDS under 40 KB, and the register budget that goes
-// with four wavefronts per SIMD (128) is met without spilling.  The kernel waits on memory most of its time, so a fourth
-// resident group is worth more than a larger window.
-#ifndef SRF_FUSED_WAVES_PER_EU
-#define SRF_FUSED_WAVES_PER_EU 4
-#endif
-#define SRF_FUSED_OCCUPANCY __attribute__((amdgpu_waves_per_eu(SRF_FUSED_WAVES_PER_EU, SRF_FUSED_WAVES_PER_EU)))
-template <bool HALF_IN, bool HALF_OUT>
-__global__ void __launch_bounds__(fused::THREADS) SRF_FUSED_OCCUPANCY k_composite_fused(fused::Args A, const uint32_t* __restrict__ n_rays_counter, const float* __restrict__ mean_density_ptr,
-                                                                     uint32_t n_groups, ChainScratch S, uint32_t* __restrict__ compacted_counter) {
+// Ordering point between the phases of a group (see srf_composite_fused.h): a workgroup barrier.
+__device__ __forceinline__ void group_sync() { __syncthreads(); }
+
+// ---- groups that do not fit the streaming path ------------------------------------------------
+// The streaming kernel takes groups whose rays are laid out back to back and whose samples fit one of its windows.  The
+// others (arbitrary caller-supplied offsets; more samples than one window) are rare and are kept out of its code:
+//   k_chain_prepare      clears the chain's status words, plans every group and notes how many items it makes
+//   k_chain_items        numbers the items in ray order and lists those of groups that the streaming path does not take
+//   k_slow_groups (fwd)  forward pass of the listed groups; leaves the number of samples every one of their rays consumes
+//   k_composite_stream   for a listed group only chains those counts to its neighbours' and leaves the rays' compacted offsets
+//   k_slow_groups (bwd)  forward pass again, then commit and gradients at those offsets
+// Rays not laid out back to back are composited one lane per ray; groups longer than a window run the window phases over
+// all windows.
+
+// Records of one group into a plan, by the 64 lanes of one wave: what fused::plan_lane and fused::plan_finish_lane
+// compute lane by lane through LDS, with the wave's own reductions instead (64 lanes adding to one LDS word take turns).
+__device__ __forceinline__ void plan_from_records(uint32_t lane, uint32_t g, U2 rec, const fused::Args& A, fused::Plan& pl) {
 	using namespace fused;
-	__shared__ Shared sh;
-	const uint32_t tid = threadIdx.x;
-	// Groups are numbered by workgroup index.  A group only ever waits for lower-numbered groups, and
-	// workgroups are handed to the hardware in index order, so the lowest unfinished group is always
-	// running; a shared ticket counter would give the same order but costs one same-address
-	// device-wide atomic per group, which serialises the launch.
-	const uint32_t g = blockIdx.x;
-#ifdef SRF_FUSED_TIMING
-	unsigned long long t_prev_ = clock64();
-	unsigned long long t_acc_[6] = {0, 0, 0, 0, 0, 0};
-#endif
-	Plan& pl = sh.plan;
-	if (tid == 0) { pl.misc[M_SUM] = 0; pl.misc[M_CONTIG] = 1; }
-	group_sync();
 	const uint32_t ray0 = g * RAYS;
-	const uint32_t counter_now = *n_rays_counter;
-	A.mean_density = mean_density_ptr ? *mean_density_ptr : 0.f;
-	A.n_active = A.K.n_rays;                 // the record loads do not wait for the counter ...
-	Float4 target_rgba = mk4(0.f, 0.f, 0.f, 0.f);
-	U2 rec; rec.x = 0; rec.y = 0;
-	if (tid < RAYS && ray0 + tid < A.K.n_rays) {
-		rec = *(const U2*)(A.ray_coord_indices + 2 * (size_t)(ray0 + tid));
-		target_rgba = *(const Float4*)(A.rays_rgba + 4 * (size_t)(ray0 + tid));
+	const uint32_t n_here = A.n_active > ray0 ? (A.n_active - ray0 < RAYS ? A.n_active - ray0 : RAYS) : 0;
+	const uint32_t rn = rec.x, rabs = rec.y;             // (0, 0) past the active count
+	const uint32_t s0 = n_here ? (uint32_t)__shfl((int)rabs, 0, WAVE) : 0u;
+	const uint32_t prev_rabs = (uint32_t)__shfl_up((int)rabs, 1, WAVE), prev_rn = (uint32_t)__shfl_up((int)rn, 1, WAVE);
+	const uint64_t prev_end = lane ? (uint64_t)prev_rabs + prev_rn : (uint64_t)s0;
+	const bool mine = lane < n_here;
+	const bool out_of_order = mine && (uint64_t)rabs < prev_end;
+	const uint32_t sum = wave_sum_u32(mine ? rn : 0u);
+	const uint32_t last = n_here ? n_here - 1 : 0u;
+	const uint64_t end = n_here ? (uint64_t)(uint32_t)__shfl((int)rabs, (int)last, WAVE) + (uint32_t)__shfl((int)rn, (int)last, WAVE) : 0ull;
+	const uint64_t total64 = end >= s0 ? end - s0 : 0ull;
+	const uint32_t total = total64 > 0xffffffffull ? 0xffffffffu : (uint32_t)total64;
+	const bool contiguous = __ballot(out_of_order) == 0ull && !((uint64_t)total > (uint64_t)sum + GAP_SLACK);
+	pl.rn[lane] = rn;
+	pl.rabs[lane] = rabs;
+	pl.rbase[lane] = mine ? rabs - s0 : total;
+	if (lane == 0) {
+		pl.rbase[RAYS] = total;
+		pl.misc[M_S0] = s0; pl.misc[M_TOTAL] = total; pl.misc[M_SUM] = sum; pl.misc[M_CONTIG] = contiguous ? 1u : 0u;
+		pl.misc[M_LANE_LO] = 0; pl.misc[M_LANE_HI] = RAYS; pl.misc[M_GROUP] = g;
 	}
-	A.n_active = counter_now < A.K.n_rays ? counter_now : A.K.n_rays;   // ... which only masks them
-	if (tid < RAYS) {
-		const bool live = ray0 + tid < A.n_active;
-		pl.rn[tid] = live ? rec.x : 0u;
-		pl.rabs[tid] = live ? rec.y : 0u;
-	}
-	group_sync();
-	if (tid < RAYS) plan_lane(tid, ray0, A, pl);
-	group_sync();
-	if (tid < RAYS) plan_finish_lane(tid, ray0, A, pl);
-	group_sync();
-	SRF_TSTAMP(0);
-	const bool contig = pl.misc[M_CONTIG] != 0;
-	const uint32_t total = pl.misc[M_TOTAL];
-	const uint32_t n_win = (total + WIN - 1) / WIN;
-	SlotState<HALF_IN> st;
-	RayCarry c;
-	uint32_t n_scattered = 0;
-	if (contig) {
-		if (tid < RAYS) reset_carry(tid, pl, c);
-		for (uint32_t win = 0; win < n_win; ++win) {
-			phase_a<HALF_IN>(tid, win, A, sh, pl, st);
-			group_sync();
-			SRF_TSTAMP(1);
-			if (tid < RAYS) chain(tid, win, A, sh, pl, c);
-			group_sync();
-			SRF_TSTAMP(2);
-		}
-		if (tid < RAYS) finish_ray(tid, ray0, A, sh, c, target_rgba);
-	} else if (tid < RAYS) {
-		loss_forward_body<HALF_IN>(ray0 + tid, A.K, A.rays_rgba, A.n_active, A.ray_coord_indices, A.dt_arr, A.net, &sh.fw[tid], &n_scattered, A.rgb_ray_out);
-		sh.rnf[tid] = n_scattered;
-	}
-	group_sync();
-	if (tid < WAVE) {      // first wave: ordered compacted offsets
-		const uint32_t n = tid < RAYS ? sh.rnf[tid] : 0u;
-		const uint32_t incl = wave_inclusive_scan_u32(n);
-		const uint32_t group_total = (uint32_t)__shfl((int)incl, WAVE - 1, WAVE);
-		SRF_TSTAMP(3);
-		const uint32_t prefix = chained_prefix(S, g, group_total);
-		SRF_TSTAMP(4);
-		const uint32_t cbase = prefix + incl - n;
-		if (tid < RAYS) {
-			if (contig) commit_ray(tid, ray0, cbase, A, sh);
-			else sh.out[tid].cbase = cbase;
-		}
-		if (g == n_groups - 1 && tid == 0) *compacted_counter = prefix + group_total;
-	}
-	group_sync();
-	if (contig) {
-		if (n_win == 1) {
-			phase_c<HALF_IN, HALF_OUT>(tid, 0, A, sh, pl, st);
-		} else if (n_win > 1) {
-			if (tid < RAYS) reset_carry(tid, pl, c);
-			for (uint32_t win = 0; win < n_win; ++win) {
-				phase_a<HALF_IN>(tid, win, A, sh, pl, st);
-				group_sync();
-				if (tid < RAYS) chain(tid, win, A, sh, pl, c);
-				group_sync();
-				phase_c<HALF_IN, HALF_OUT>(tid, win, A, sh, pl, st);
-				group_sync();
-			}
-		}
-	} else if (tid < RAYS) {
-		loss_backward_body<HALF_IN, HALF_OUT>(ray0 + tid, A.K, A.n_active, A.ray_coord_indices, A.dt_arr, A.coords, A.compacted_coords, A.net, A.dloss, A.loss_output,
-		                                      A.mean_density, sh.fw[tid], sh.rnf[tid], sh.out[tid].cbase, nullptr);
-	}
-	SRF_TSTAMP(5);
-#ifdef SRF_FUSED_TIMING
-	if (tid == 0) {
-		unsigned long long* slot = S.timing + (size_t)(g & 1023u) * 8;
-		for (int k = 0; k < 6; ++k) atomicAdd(slot + k, t_acc_[k]);
-		atomicAdd(slot + 7, 1ull);
-	}
-#endif
+	__builtin_amdgcn_wave_barrier();
 }
 
-// ------------------------------------------------------------------------------------
-// Two-pass training compositing.  Pass 1 (BACKWARD = false) runs the forward phases of every group
-// and leaves the number of samples each ray consumed; a device-wide exclusive scan turns those into
-// ordered compacted offsets; pass 2 (BACKWARD = true) runs the forward phases again and emits
-// gradients at those offsets.  No workgroup ever waits for another, so a slow group (a very long
-// ray) delays nobody, at the price of reading the samples twice.
-//
-// Each workgroup walks over many groups (g, g + gridDim.x, ...) and keeps the memory system busy
-// while it computes: the ray records of the group after next and the samples of the next group are
-// requested before the current group's chain starts, and are only needed one iteration later.  The
-// two register sets X and Y swap roles every iteration, so nothing in flight is ever copied.
-// ------------------------------------------------------------------------------------
-template <bool HALF_IN>
-struct PassRegs {
-	fused::SlotState<HALF_IN> st;   // samples of the group being worked on / being fetched
-	U2 rec;                         // (count, offset) of one ray of the group after
-	Float4 target;
-	uint32_t cbase;
+__device__ __forceinline__ U2 load_record(uint32_t g, uint32_t lane, const fused::Args& A) {
+	U2 rec; rec.x = 0; rec.y = 0;
+	const uint32_t i = g * fused::RAYS + lane;
+	if (i < A.n_active) rec = *(const U2*)(A.ray_coord_indices + 2 * (size_t)i);
+	return rec;
+}
+
+// One wave per group, PREPARE_WAVES groups per workgroup; a workgroup also leaves the number of items its groups make.
+__global__ void __launch_bounds__(PREPARE_WAVES * WAVE) k_chain_prepare(fused::Args A, const uint32_t* __restrict__ n_rays_counter, ChainScratch S, uint32_t n_groups_max,
+                                                                       const uint32_t* __restrict__ counter) {
+	using namespace fused;
+	__shared__ Plan plans[PREPARE_WAVES];
+	__shared__ uint32_t n_items_of_wave[PREPARE_WAVES];
+	const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+	const uint32_t g = blockIdx.x * PREPARE_WAVES + wave;
+	if (blockIdx.x == 0 && threadIdx.x == 0) { *S.initial = *counter; *S.error = 0u; *S.slow_count = 0u; }
+	if (g < n_groups_max) {
+		if (lane < 2) S.item_status[2 * g + lane] = 0ull;
+		if (lane == 0 && g % 32 == 0) { S.seg_status[(size_t)(g / 32) * SEG_STRIDE] = 0ull; S.seg_prefix[g / 32] = 0ull; }
+	}
+	const uint32_t counter_now = *n_rays_counter;
+	A.n_active = counter_now < A.K.n_rays ? counter_now : A.K.n_rays;
+	uint32_t word = 0;
+	if (g < div_up(A.n_active, RAYS)) {
+		Plan& pl = plans[wave];
+		plan_from_records(lane, g, load_record(g, lane, A), A, pl);
+		word = group_items_word<StreamGeometry>(pl);
+		if (lane == 0) S.group_words[g] = word;
+	}
+	if (lane == 0) n_items_of_wave[wave] = word & 0xffu;
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		uint32_t n = 0;
+		for (uint32_t k = 0; k < PREPARE_WAVES; ++k) n += n_items_of_wave[k];
+		S.prepare_sums[blockIdx.x] = n;
+	}
+}
+
+// Numbers the items: an exclusive scan of the groups' item counts.  A workgroup takes ITEMS_THREADS consecutive groups (one
+// per thread); what lies before them it adds up from the sums that k_chain_prepare's workgroups left.
+constexpr uint32_t ITEMS_THREADS = 1024;
+static_assert(ITEMS_THREADS % PREPARE_WAVES == 0, "an items workgroup starts where a prepare workgroup starts");
+__global__ void __launch_bounds__(ITEMS_THREADS) k_chain_items(uint32_t n_rays_max, const uint32_t* __restrict__ n_rays_counter, ChainScratch S) {
+	using namespace fused;
+	__shared__ uint32_t wave_total[ITEMS_THREADS / WAVE], wave_before[ITEMS_THREADS / WAVE];
+	const uint32_t tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+	const uint32_t counter_now = *n_rays_counter;
+	const uint32_t n_groups = div_up(counter_now < n_rays_max ? counter_now : n_rays_max, RAYS);
+	const uint32_t g_first = blockIdx.x * ITEMS_THREADS;
+	if (g_first >= n_groups && !(n_groups == 0 && blockIdx.x == 0)) return;
+	const uint32_t g = g_first + tid;
+	const uint32_t word = g < n_groups ? S.group_words[g] : 0u;
+	uint32_t before = 0;
+	for (uint32_t k = tid; k < g_first / PREPARE_WAVES; k += ITEMS_THREADS) before += S.prepare_sums[k];
+	const uint32_t n = word & 0xffu;
+	const uint32_t incl = wave_inclusive_scan_u32(n);
+	const uint32_t before_w = wave_sum_u32(before);
+	if (lane == WAVE - 1) { wave_total[wave] = incl; wave_before[wave] = before_w; }
+	__syncthreads();
+	uint32_t base = 0, all = 0;
+	for (uint32_t k = 0; k < ITEMS_THREADS / WAVE; ++k) { const uint32_t t = wave_total[k]; base += wave_before[k] + (k < wave ? t : 0u); all += wave_before[k] + t; }
+	if (n != 0) {
+		const uint32_t first = base + incl - n;
+		U2 it[2];
+		items_of_group(g, word, it);
+		S.items[first] = it[0];
+		if (n == 2) S.items[first + 1] = it[1];
+		if (item_listed(it[0])) S.slow_items[atomicAdd(S.slow_count, 1u)] = first;
+	}
+	if (tid == 0 && g_first + ITEMS_THREADS >= n_groups) *S.n_items = all;     // the workgroup with the last group
+}
+
+struct SlowShared {
+	fused::Window<fused::WideGeometry> w;
+	fused::RayLds rl;
+	fused::Plan plan;
 };
 
-template <bool HALF_IN, bool BACKWARD>
-__device__ inline void pass_load_rec(uint32_t tid, uint32_t g, uint32_t n_groups, const fused::Args& A, U2& rec) {
-	using namespace fused;
-	rec.x = 0; rec.y = 0;
-	const uint32_t i = g * RAYS + tid;
-	if (g < n_groups && tid < RAYS && i < A.K.n_rays) rec = *(const U2*)(A.ray_coord_indices + 2 * (size_t)i);
-}
-
-// plan of group g from the records its lanes hold; returns nothing, leaves pl ready after the last barrier
-__device__ inline void pass_plan(uint32_t tid, uint32_t g, const fused::Args& A, fused::Plan& pl, U2 rec) {
-	using namespace fused;
-	const uint32_t ray0 = g * RAYS;
-	if (tid == 0) { pl.misc[M_SUM] = 0; pl.misc[M_CONTIG] = 1; }
-	if (tid < RAYS) {
-		const bool live = ray0 + tid < A.n_active;
-		pl.rn[tid] = live ? rec.x : 0u;
-		pl.rabs[tid] = live ? rec.y : 0u;
-	}
-	group_sync();
-	if (tid < RAYS) plan_lane(tid, ray0, A, pl);
-	group_sync();
-	if (tid < RAYS) plan_finish_lane(tid, ray0, A, pl);
-	group_sync();
-}
-
-// requests everything group gn needs except its records: the samples of its first window, targets, offsets
-template <bool HALF_IN, bool BACKWARD>
-__device__ __forceinline__ void pass_fetch_group(uint32_t tid, uint32_t gn, const fused::Args& A, const fused::Plan& pn, const uint32_t* __restrict__ cbase_arr,
-                                                 PassRegs<HALF_IN>& R) {
-	using namespace fused;
-	if (pn.misc[M_CONTIG] != 0 && pn.misc[M_TOTAL] <= WIN) phase_a_load<HALF_IN>(tid, 0, A, pn, R.st);
-	const uint32_t i = gn * RAYS + tid;
-	R.target = mk4(0.f, 0.f, 0.f, 0.f);
-	R.cbase = 0;
-	if (tid < RAYS && i < A.K.n_rays) {
-		R.target = *(const Float4*)(A.rays_rgba + 4 * (size_t)i);
-		if (BACKWARD) R.cbase = cbase_arr[i];
-	}
-}
-
-// groups that do not fit the fast path (rays not laid out back to back, or more samples than one window) are put on a
-// list by the forward pass and handled by a kernel of their own, so that they cost the fast path neither registers nor size
 template <bool HALF_IN, bool HALF_OUT, bool BACKWARD>
-__device__ __forceinline__ void pass_slow_group(uint32_t tid, uint32_t gi, const fused::Args& A, fused::Shared& sh, fused::Plan& pl, Float4 target, uint32_t cbase, uint32_t* n_fwd) {
+__global__ void __launch_bounds__(fused::WideGeometry::THREADS) k_slow_groups(fused::Args A, const uint32_t* __restrict__ n_rays_counter, const float* __restrict__ mean_density_ptr, ChainScratch S) {
 	using namespace fused;
-	const uint32_t ray0 = gi * RAYS;
-	if (pl.misc[M_CONTIG] != 0) {
-		const uint32_t n_win = (pl.misc[M_TOTAL] + WIN - 1) / WIN;
-		SlotState<HALF_IN> st;
-		RayCarry c;
-		if (tid < RAYS) reset_carry(tid, pl, c);
-		for (uint32_t win = 0; win < n_win; ++win) {
-			phase_a<HALF_IN>(tid, win, A, sh, pl, st);
-			group_sync();
-			if (tid < RAYS) chain(tid, win, A, sh, pl, c);
-			group_sync();
-		}
-		if (tid < RAYS) finish_ray(tid, ray0, A, sh, c, target);
-		if (BACKWARD) {
-			if (tid < RAYS) commit_ray(tid, ray0, cbase, A, sh);
-			group_sync();
-			if (tid < RAYS) reset_carry(tid, pl, c);
-			for (uint32_t win = 0; win < n_win; ++win) {
-				phase_a<HALF_IN>(tid, win, A, sh, pl, st);
-				group_sync();
-				if (tid < RAYS) chain(tid, win, A, sh, pl, c);
-				group_sync();
-				phase_c<HALF_IN, HALF_OUT>(tid, win, A, sh, pl, st);
-				group_sync();
-			}
-		} else if (tid < RAYS && ray0 + tid < A.K.n_rays) {
-			n_fwd[ray0 + tid] = sh.rnf[tid];
-		}
-	} else if (tid < RAYS) {
-		uint32_t n = 0;
-		loss_forward_body<HALF_IN>(ray0 + tid, A.K, A.rays_rgba, A.n_active, A.ray_coord_indices, A.dt_arr, A.net, &sh.fw[tid], &n, A.rgb_ray_out);
-		if (BACKWARD) {
-			loss_backward_body<HALF_IN, HALF_OUT>(ray0 + tid, A.K, A.n_active, A.ray_coord_indices, A.dt_arr, A.coords, A.compacted_coords, A.net, A.dloss, A.loss_output,
-			                                      A.mean_density, sh.fw[tid], n, cbase, nullptr);
-		} else if (ray0 + tid < A.K.n_rays) {
-			n_fwd[ray0 + tid] = n;
-		}
-	}
-}
-
-// one group: cur holds its data, nxt.rec the records of the next group; on return the register sets have swapped roles
-template <bool HALF_IN, bool HALF_OUT, bool BACKWARD>
-__device__ __forceinline__ void pass_iteration(uint32_t tid, uint32_t gi, uint32_t stride, uint32_t n_groups, const fused::Args& A, fused::Shared& sh,
-                                               fused::Plan& pl, fused::Plan& pn, PassRegs<HALF_IN>& cur, PassRegs<HALF_IN>& nxt,
-                                               uint32_t* __restrict__ n_fwd, const uint32_t* __restrict__ cbase_arr, uint32_t* __restrict__ slow_list
-#ifdef SRF_FUSED_TIMING
-                                               , unsigned long long* t_acc_, unsigned long long& t_prev_
-#endif
-                                               ) {
-	using namespace fused;
-	const uint32_t ray0 = gi * RAYS;
-	const uint32_t total = pl.misc[M_TOTAL];
-	const bool fast = pl.misc[M_CONTIG] != 0 && total <= WIN;
-	SRF_TSTAMP(0);
-	if (fast && total > 0) phase_a_compute<HALF_IN>(tid, 0, A, sh, pl, cur.st);
-	SRF_TSTAMP(1);
-	// the next group: plan it and request its data; the records of the group after it go where this group's were
-	const uint32_t gn = gi + stride;
-	if (gn < n_groups) {
-		pass_plan(tid, gn, A, pn, nxt.rec);
-		pass_fetch_group<HALF_IN, BACKWARD>(tid, gn, A, pn, cbase_arr, nxt);
-		pass_load_rec<HALF_IN, BACKWARD>(tid, gn + stride, n_groups, A, cur.rec);
-	} else {
-		group_sync();
-	}
-	SRF_TSTAMP(2);
-	if (fast) {
-		RayCarry c;
-		if (tid < RAYS) {
-			reset_carry(tid, pl, c);
-			if (total > 0) chain(tid, 0, A, sh, pl, c);
-			finish_ray(tid, ray0, A, sh, c, cur.target);
-			if (BACKWARD) commit_ray(tid, ray0, cur.cbase, A, sh);
-			else if (ray0 + tid < A.K.n_rays) n_fwd[ray0 + tid] = sh.rnf[tid];
-		}
-		SRF_TSTAMP(3);
-		if (BACKWARD) {
-			group_sync();
-			if (total > 0) phase_c<HALF_IN, HALF_OUT>(tid, 0, A, sh, pl, cur.st);
-		}
-		SRF_TSTAMP(4);
-	} else if (!BACKWARD && tid == 0) {
-		slow_list[1 + atomicAdd(slow_list, 1u)] = gi;     // the backward pass walks the same list
-	}
-	group_sync();
-	SRF_TSTAMP(5);
-}
-
-// the listed groups, one workgroup at a time, nothing prefetched
-template <bool HALF_IN, bool HALF_OUT, bool BACKWARD>
-__global__ void __launch_bounds__(fused::THREADS) k_composite_pass_slow(fused::Args A_in, const uint32_t* __restrict__ n_rays_counter, const float* __restrict__ mean_density_ptr,
-                                                                         uint32_t* __restrict__ n_fwd, const uint32_t* __restrict__ cbase_arr, const uint32_t* __restrict__ slow_list) {
-	using namespace fused;
-	__shared__ Shared sh;
-	const uint32_t tid = threadIdx.x;
-	const uint32_t n_listed = slow_list[0];
+	using G = WideGeometry;
+	__shared__ SlowShared sh;
+	const uint32_t tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+	const uint32_t n_listed = *S.slow_count;
 	if (blockIdx.x >= n_listed) return;
 	const uint32_t counter_now = *n_rays_counter;
-	Args A = A_in;
 	A.mean_density = mean_density_ptr ? *mean_density_ptr : 0.f;
 	A.n_active = counter_now < A.K.n_rays ? counter_now : A.K.n_rays;
+	if (!BACKWARD) A.rgb_ray_out = nullptr;      // written once, by the second forward pass
+	Plan& pl = sh.plan;
 	for (uint32_t k = blockIdx.x; k < n_listed; k += gridDim.x) {
-		const uint32_t g = slow_list[1 + k];
-		U2 rec;
-		pass_load_rec<HALF_IN, BACKWARD>(tid, g, 0xffffffffu, A, rec);
-		pass_plan(tid, g, A, sh.plan, rec);
-		const uint32_t i = g * RAYS + tid;
-		Float4 target = mk4(0.f, 0.f, 0.f, 0.f);
-		uint32_t cbase = 0;
-		if (tid < RAYS && i < A.K.n_rays) {
-			target = *(const Float4*)(A.rays_rgba + 4 * (size_t)i);
-			if (BACKWARD) cbase = cbase_arr[i];
+		const uint32_t g = S.items[S.slow_items[k]].x;
+		const uint32_t ray0 = g * RAYS;
+		if (wave == 0) plan_from_records(lane, g, load_record(g, lane, A), A, pl);
+		group_sync();
+		const bool live = wave == 0 && ray0 + lane < A.n_active;
+		if (pl.misc[M_CONTIG] != 0) {
+			const uint32_t n_win = (pl.misc[M_TOTAL] + G::WIN - 1) / G::WIN;
+			SlotState<G, HALF_IN> st;
+			RayCarry c;
+			Float4 target = mk4(0.f, 0.f, 0.f, 0.f);
+			if (live) target = *(const Float4*)(A.rays_rgba + 4 * (size_t)(ray0 + lane));
+			if (wave == 0) reset_carry(lane, pl, c);
+			for (uint32_t win = 0; win < n_win; ++win) {
+				phase_a<G, HALF_IN>(tid, win, A, sh.w, pl, st);
+				group_sync();
+				if (wave == 0) chain<G>(lane, win, A, sh.w, sh.rl, pl, c);
+				group_sync();
+			}
+			if (wave == 0) finish_ray(lane, ray0, A, sh.rl, c, target);
+			if (!BACKWARD) {
+				if (live) S.side[ray0 + lane] = sh.rl.rnf[lane];
+			} else {
+				if (wave == 0) commit_ray(lane, ray0, live ? S.side[ray0 + lane] : 0u, A, sh.rl);
+				group_sync();
+				if (wave == 0) reset_carry(lane, pl, c);
+				for (uint32_t win = 0; win < n_win; ++win) {
+					phase_a<G, HALF_IN>(tid, win, A, sh.w, pl, st);
+					group_sync();
+					if (wave == 0) chain<G>(lane, win, A, sh.w, sh.rl, pl, c);
+					group_sync();
+					phase_c<G, HALF_IN, HALF_OUT>(tid, win, A, sh.w, sh.rl, pl, st);
+					group_sync();
+				}
+			}
+		} else if (wave == 0) {
+			uint32_t n = 0;
+			FwdRay fw;
+			loss_forward_body<HALF_IN>(ray0 + lane, A.K, A.rays_rgba, A.n_active, A.ray_coord_indices, A.dt_arr, A.net, &fw, &n, A.rgb_ray_out);
+			if (!BACKWARD) {
+				if (live) S.side[ray0 + lane] = n;
+			} else if (live) {
+				loss_backward_body<HALF_IN, HALF_OUT>(ray0 + lane, A.K, A.n_active, A.ray_coord_indices, A.dt_arr, A.coords, A.compacted_coords, A.net, A.dloss, A.loss_output,
+				                                      A.mean_density, fw, n, S.side[ray0 + lane], nullptr);
+			}
 		}
-		pass_slow_group<HALF_IN, HALF_OUT, BACKWARD>(tid, g, A, sh, sh.plan, target, cbase, n_fwd);
 		group_sync();
 	}
 }
 
-template <bool HALF_IN, bool HALF_OUT, bool BACKWARD>
-__global__ void __launch_bounds__(fused::THREADS) k_composite_pass(fused::Args A_in, const uint32_t* __restrict__ n_rays_counter, const float* __restrict__ mean_density_ptr,
-                                                                    uint32_t n_groups, uint32_t* __restrict__ n_fwd, const uint32_t* __restrict__ cbase_arr, uint32_t* __restrict__ slow_list, unsigned long long* timing) {
-	using namespace fused;
-	__shared__ Shared sh;
-	__shared__ Plan plan_next;   // the group being fetched while the current one is worked on
-	const uint32_t tid = threadIdx.x;
-	const uint32_t stride = gridDim.x;
-	const uint32_t counter_now = *n_rays_counter;
-	Args A = A_in;
-	A.mean_density = mean_density_ptr ? *mean_density_ptr : 0.f;
-	A.n_active = counter_now < A.K.n_rays ? counter_now : A.K.n_rays;
-	uint32_t g = blockIdx.x;
-	if (g >= n_groups) return;
-	PassRegs<HALF_IN> X, Y;
-#ifdef SRF_FUSED_TIMING
-	unsigned long long t_prev_ = clock64();
-	unsigned long long t_acc_[6] = {0, 0, 0, 0, 0, 0};
-	unsigned long long n_iter_ = 0;
-#define SRF_TARGS , t_acc_, t_prev_
+// ---- the streaming kernel ---------------------------------------------------------------------
+// Workgroups are persistent: workgroup b works on items b, b + gridDim.x, b + 2 gridDim.x, ...  (Handing the items out
+// in the order in which workgroups become free would need a counter that every item increments, and the device serialises
+// those increments at a rate below the rate of items; consecutive items on one workgroup would make each workgroup wait
+// for its neighbour's last item.)  A workgroup's first wave walks
+// rays (one lane per ray: count, chain, finish, ordered offsets), its second wave plans, its other waves work on samples
+// (phases A and C), and three items are under way at any time, in two LDS windows:
+//
+//                 first half of iteration j                      second half of iteration j
+//   ray wave      look-back and commit of item j                 count of item j + 1 (its total is published), then its chain
+//   plan wave     finish of item j (colours, loss, its gradient) plan of item j + 3; records further ahead requested; losses of
+//                                                                item j written; coordinates of item j's kept samples moved
+//   sample waves  phase A of item j + 1 (other window)           samples of item j + 2 requested; phase C of item j
+//
+// so every load has at least half an iteration to arrive before it is used, and an item's total is published a chain and
+// a barrier before its own look-back needs its predecessors' totals: a workgroup has to fall that far behind the others
+// before they wait for it.  The ray wave is the one sequential stream of a workgroup, so it runs at raised
+// priority.  An item waits for every lower-numbered item's total.  Lower-numbered items belong to workgroups that are
+// resident at the same time (the grid is sized to what the device holds at once); waits are bounded all the same.
+// Two workgroups per CU (two windows take most of their 80 KB of LDS each).
+#define SRF_STREAM_OCCUPANCY __attribute__((amdgpu_waves_per_eu(4, 4)))
+constexpr uint32_t STREAM_WORKGROUPS_PER_CU = 2;
+// Eight waves per workgroup: the hardware deals a workgroup's waves round the four SIMDs, so two such workgroups fill every
+// SIMD evenly (a workgroup of, say, six waves may not find room next to another although the totals fit, and the items of a
+// workgroup that is not resident are waited for in vain).
+constexpr uint32_t STREAM_THREADS = 2 * WAVE + fused::StreamGeometry::THREADS;
+static_assert(STREAM_THREADS == 8 * WAVE, "workgroup shape");
+
+struct StreamShared {
+	fused::Window<fused::StreamGeometry> win[2];
+	fused::RayLds rl;
+	fused::Plan plan[fused::NPLAN];     // ring: the plans of the three items under way and of the one after them
+	fused::Plan group_plan;             // plan wave: the group whose rays the item being planned belongs to
+};
+
+// Build flag SRF_STREAM_TIMING: lane 0 of the ray wave and of the first sample wave add up the cycles they spend in
+// the parts of an iteration, into counters after the chain's misc words.
+#ifdef SRF_STREAM_TIMING
+#define SRF_T(k) do { if (lane == 0 && wave <= 2) { const unsigned long long now_ = clock64(); t_acc_[k] += now_ - t_prev_; t_prev_ = now_; } } while (0)
 #else
-#define SRF_TARGS
+#define SRF_T(k) ((void)0)
 #endif
-	// prologue: the first group's records, plan and data; the second group's records
-	pass_load_rec<HALF_IN, BACKWARD>(tid, g, n_groups, A, X.rec);
-	pass_plan(tid, g, A, sh.plan, X.rec);
-	pass_fetch_group<HALF_IN, BACKWARD>(tid, g, A, sh.plan, cbase_arr, X);
-	pass_load_rec<HALF_IN, BACKWARD>(tid, g + stride, n_groups, A, Y.rec);
-	for (;;) {
-		pass_iteration<HALF_IN, HALF_OUT, BACKWARD>(tid, g, stride, n_groups, A, sh, sh.plan, plan_next, X, Y, n_fwd, cbase_arr, slow_list SRF_TARGS);
-		g += stride;
-#ifdef SRF_FUSED_TIMING
-		n_iter_ += 2;
+
+template <bool HALF_IN, bool HALF_OUT, bool PLAIN>
+__global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composite_stream(fused::Args A, const uint32_t* __restrict__ n_rays_counter, const float* __restrict__ mean_density_ptr,
+                                                                     ChainScratch S, uint32_t* __restrict__ compacted_counter) {
+	using namespace fused;
+	using G = StreamGeometry;
+	static_assert(RAYS == WAVE, "one lane per ray");
+	static_assert(NPLAN == 4, "three items under way, one being planned");
+	__shared__ StreamShared sh;
+	const uint32_t tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+	const uint32_t st_id = tid - 2 * WAVE;                   // index among the sample threads (waves 2-7)
+	const bool ray_wave = wave == 0, plan_wave = wave == 1;
+	const uint32_t counter_now = *n_rays_counter;
+	A.mean_density = mean_density_ptr ? *mean_density_ptr : 0.f;
+	A.n_active = counter_now < A.K.n_rays ? counter_now : A.K.n_rays;   // rays past the active count belong to no item: they are left untouched
+	const uint32_t n_items = *S.n_items;
+	if (blockIdx.x >= n_items) return;
+
+#ifdef SRF_STREAM_TIMING
+	unsigned long long t_acc_[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+	unsigned long long t_prev_ = clock64();
+	unsigned long long n_it_ = 0;
+	bool t_on_ = false;
 #endif
-		if (g >= n_groups) break;
-		pass_iteration<HALF_IN, HALF_OUT, BACKWARD>(tid, g, stride, n_groups, A, sh, plan_next, sh.plan, Y, X, n_fwd, cbase_arr, slow_list SRF_TARGS);
-		g += stride;
-		if (g >= n_groups) break;
+	SlotState<G, HALF_IN> set_c, set_a, set_l;     // samples of the item in phase C / in phase A / being loaded
+	// ray wave, about the item it commits in the next first half
+	uint32_t n_cur = 0, incl_cur = 0;               // count of its ray, scanned over the wave
+	uint32_t total_cur = 0;                         // samples it keeps
+	ChainPeek peek;
+	peek.vg = 0ull; peek.vs = 0ull; peek.vp = 0ull; peek.initial = 0u;
+	RayCarry carry;
+	carry.T = 1.f; carry.Cr = 0.f; carry.Cg = 0.f; carry.Cb = 0.f; carry.k = 0; carry.numsteps = 0; carry.done = 0;
+	// plan wave: the numbers of the workgroup's items, in the order it takes them ...
+	uint32_t handed = 0;
+	auto next_number = [&]() -> uint32_t {
+		const uint64_t i = (uint64_t)blockIdx.x + (uint64_t)handed * gridDim.x;
+		if (i >= n_items) return NO_ITEM;
+		++handed;
+		return (uint32_t)i;
+	};
+	// ... the item it plans next (number, record, its group's ray records: requested an iteration earlier) and the item after that,
+	// and the target colours of the rays it finishes next
+	Float4 target = mk4(0.f, 0.f, 0.f, 0.f);
+	uint32_t number_p = NO_ITEM, number_q = NO_ITEM;
+	U2 item_p, item_q, rec_p;
+	item_p.x = 0; item_p.y = 0; item_q = item_p; rec_p = item_p;
+	auto load_item = [&](uint32_t number) { U2 item; item.x = 0; item.y = 0; if (number != NO_ITEM) item = S.items[number]; return item; };
+	auto plan_next = [&](Plan& out) {                // turns item_p into a plan and moves the requests one item on
+		const U2 item = item_p, rec = rec_p;
+		const uint32_t number = number_p;
+		if (number != NO_ITEM) {
+			const uint32_t g = item.x;
+#ifdef SRF_STREAM_TIMING
+			{ U2 r_ = rec; asm volatile("" : "+v"(r_.x), "+v"(r_.y)); if (lane == 0 && wave == 1 && t_on_) { const unsigned long long now_ = clock64(); t_acc_[5] += now_ - t_prev_; t_prev_ = now_; } }
+#endif
+			plan_from_records(lane, g, rec, A, sh.group_plan);
+#ifdef SRF_STREAM_TIMING
+			if (lane == 0 && wave == 1 && t_on_) { const unsigned long long now_ = clock64(); t_acc_[6] += now_ - t_prev_; t_prev_ = now_; }
+#endif
+			plan_part_lane(lane, sh.group_plan, item_lo(item), item_hi(item), g, out);
+#ifdef SRF_STREAM_TIMING
+			if (lane == 0 && wave == 1 && t_on_) { const unsigned long long now_ = clock64(); t_acc_[7] += now_ - t_prev_; t_prev_ = now_; }
+#endif
+		}
+		if (lane == 0) {
+			out.misc[M_ITEM] = number;
+			if (number != NO_ITEM && item_listed(item)) out.misc[M_CONTIG] = 0;     // only its offsets pass through here
+		}
+		item_p = item_q; number_p = number_q;
+		rec_p = load_record(item_p.x, lane, A);     // (no item: group 0's, unused)
+		number_q = next_number();
+		item_q = load_item(number_q);
+	};
+	if (plan_wave) {
+		number_p = next_number(); item_p = load_item(number_p);
+		number_q = next_number(); item_q = load_item(number_q);
+		rec_p = load_record(item_p.x, lane, A);
+		plan_next(sh.plan[0]);
 	}
-#ifdef SRF_FUSED_TIMING
-	if (tid == 0 && timing) {
-		unsigned long long* slot = timing + (size_t)(blockIdx.x & 1023u) * 8;
-		for (int k = 0; k < 6; ++k) atomicAdd(slot + k, t_acc_[k]);
-		atomicAdd(slot + 7, n_iter_);
+	group_sync();
+	if (ray_wave) __builtin_amdgcn_s_setprio(3);
+
+	// the workgroup's item `it` is finished and gets its phase C in iteration `it`; its items it + 1 and it + 2 are under way behind it
+	for (int it = -2;; ++it) {
+		const Plan& pl = sh.plan[(uint32_t)(it + 4) % NPLAN];
+		const Plan& pl1 = sh.plan[(uint32_t)(it + 5) % NPLAN];
+		const Plan& pl2 = sh.plan[(uint32_t)(it + 6) % NPLAN];
+		Plan& pl3 = sh.plan[(uint32_t)(it + 7) % NPLAN];
+		Window<G>& w = sh.win[(uint32_t)(it + 4) % 2];
+		Window<G>& w1 = sh.win[(uint32_t)(it + 5) % 2];
+		// numbers of the items (plans of items it and it + 1 were written an iteration or more ago)
+		const uint32_t i_0 = it >= 0 ? SRF_UNIFORM_U32(pl.misc[M_ITEM]) : NO_ITEM, i_1 = it + 1 >= 0 ? SRF_UNIFORM_U32(pl1.misc[M_ITEM]) : NO_ITEM;
+		const bool has0 = i_0 != NO_ITEM, has1 = i_1 != NO_ITEM;
+		const bool fast = has0 && pl.misc[M_CONTIG] != 0;
+		const bool fast1 = has1 && pl1.misc[M_CONTIG] != 0;
+		const uint32_t ray0 = has0 ? pl.misc[M_GROUP] * RAYS : 0u, lo = has0 ? pl.misc[M_LANE_LO] : 0u, hi = has0 ? pl.misc[M_LANE_HI] : 0u;
+#ifdef SRF_STREAM_TIMING
+		if (lane == 0 && wave <= 2) { ++n_it_; t_prev_ = clock64(); t_on_ = true; }
+#endif
+		// ---- first half
+		if (ray_wave) {
+			// The counter that covers memory operations cannot tell loads from stores, which complete in no fixed order, so once a
+			// store is under way every wait for a load becomes a wait for everything.  The status words requested in the previous
+			// second half are therefore waited for here, before this half's first store, while everything under way is old.
+			if (has0) asm volatile("" : "+v"(peek.vg), "+v"(peek.vs), "+v"(peek.vp), "+v"(peek.initial));
+			if (has0) {
+				const uint32_t prefix = chain_resolve(S, i_0, total_cur, peek);
+				SRF_T(6);
+				const uint32_t cbase = prefix == CHAIN_FAILED ? CHAIN_FAILED : prefix + incl_cur - n_cur;
+				if (fast) commit_ray(lane, ray0, cbase, A, sh.rl, lo, hi, false);
+				else if (ray0 + lane < A.n_active) S.side[ray0 + lane] = cbase;
+				if (i_0 == n_items - 1 && lane == 0) *compacted_counter = prefix == CHAIN_FAILED ? CHAIN_FAILED : prefix + total_cur;
+			}
+		} else if (plan_wave) {
+			if (fast) {
+				carry_from_lds(lane, sh.rl, pl, carry);
+				finish_ray(lane, ray0, A, sh.rl, carry, target, lo, hi);
+			}
+		} else {
+#ifdef SRF_STREAM_TIMING
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+			SRF_T(4);
+#endif
+			if (fast1) phase_a_compute<G, HALF_IN, PLAIN>(st_id, 0, A, w1, pl1, set_a);
+			SRF_T(5);
+		}
+		SRF_T(0);
+		group_sync();
+		SRF_T(1);
+		const bool has2 = SRF_UNIFORM_U32(pl2.misc[M_ITEM]) != NO_ITEM;      // written in the previous second half (or before the loop)
+		// ---- second half
+		if (ray_wave) {
+			if (has1) {
+				const uint32_t ray1 = pl1.misc[M_GROUP] * RAYS, lo1 = pl1.misc[M_LANE_LO], hi1 = pl1.misc[M_LANE_HI];
+				if (fast1) n_cur = count_lane<G>(lane, wave_max_u32(pl1.rn[lane]), A, w1, pl1);
+				else n_cur = (ray1 + lane < A.n_active && lane >= lo1 && lane < hi1) ? S.side[ray1 + lane] : 0u;
+				incl_cur = wave_inclusive_scan_u32(n_cur);
+				total_cur = (uint32_t)__shfl((int)incl_cur, WAVE - 1, WAVE);
+				chain_publish(S, i_1, total_cur);
+				SRF_T(7);
+				if (fast1) chain_counted<G>(lane, n_cur, wave_max_u32(n_cur), w1, sh.rl, pl1, carry);
+				peek = chain_peek(S, i_1);                            // needed in the next first half; the items before this one have published by now unless their workgroups lag
+				SRF_T(4);
+			}
+		} else if (plan_wave) {
+			// the plan first: it waits for records requested an iteration ago, and that wait must not include anything younger (see above)
+			plan_next(pl3);
+			SRF_T(4);
+			if (has1) {
+				const uint32_t ray1 = pl1.misc[M_GROUP] * RAYS;
+				if (ray1 + lane < A.n_active) target = *(const Float4*)(A.rays_rgba + 4 * (size_t)(ray1 + lane));
+			}
+			if (fast) commit_loss(lane, ray0, A, sh.rl, lo, hi);
+			if (fast) coords_copy_single<G>(lane, A, w, sh.rl, pl);
+		} else {
+			if (has2 && pl2.misc[M_CONTIG] != 0) phase_a_load_single<G, HALF_IN>(st_id, A, pl2, set_l);
+			SRF_T(7);
+			if (fast) phase_c<G, HALF_IN, HALF_OUT, PLAIN, false>(st_id, 0, A, w, sh.rl, pl, set_c);
+			SRF_T(8);
+		}
+		SRF_T(2);
+		group_sync();
+		SRF_T(3);
+		if (!has1 && !has2 && it + 1 >= 0) break;
+		set_c = set_a;
+		set_a = set_l;
+	}
+#ifdef SRF_STREAM_TIMING
+	if (lane == 0 && wave <= 2) {
+		unsigned long long* out = (unsigned long long*)(S.initial + 16) + wave * 12;
+		for (int k = 0; k < 11; ++k) atomicAdd(out + k, t_acc_[k]);
+		atomicAdd(out + 11, n_it_);
 	}
 #endif
-#undef SRF_TARGS
 }
 
 // testbed.cu:423-446 — classification of a ray: 1 alive, 2 finished with visible alpha, 0 dropped
@@ -553,6 +665,94 @@ __global__ void __launch_bounds__(256) k_fill_rollover_rescale(uint32_t n_elemen
 	net_store<HALF>(buf, i, v * (float)n_in / (float)n_elements);
 }
 
+// The chain of a streaming launch gave up (see chain_resolve): the outputs of that call are invalid.  Reported once, by the
+// first call that notices; from then on the marcher composites with the three-launch implementation, which has no waits
+// between workgroups.
+static int check_chain_error(srf_marcher* m) {
+	if (m->host_error && *m->host_error) {
+		*m->host_error = 0u;
+		m->degraded = true;
+		SRF_FAIL(SRF_ERR_HIP, "compositing: in an earlier call a workgroup gave up waiting for its predecessors' sample counts; that call's compacted "
+		                      "offsets and gradients are invalid (its compacted counter reads 0xffffffff). This marcher now uses the three-launch implementation.");
+	}
+	return SRF_OK;
+}
+
+// Workgroups of the streaming kernel that the device holds at once: the kernel's groups wait for one another, so its grid
+// must not exceed that.  Asked of the runtime once per kernel variant.
+template <bool HI, bool HO, bool PL>
+static int stream_resident_workgroups(uint32_t* out) {
+	static uint32_t cached = 0;   // per variant; the library drives one device per process
+	if (!cached) {
+		hipDeviceProp_t prop; int dev = 0, per_cu = 0;
+		SRF_HIP(hipGetDevice(&dev));
+		SRF_HIP(hipGetDeviceProperties(&prop, dev));
+		SRF_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k_composite_stream<HI, HO, PL>, (int)STREAM_THREADS, 0));
+		if (per_cu < 1) SRF_FAIL(SRF_ERR_HIP, "compositing: the streaming kernel does not fit this device");
+		if (per_cu > (int)STREAM_WORKGROUPS_PER_CU) per_cu = (int)STREAM_WORKGROUPS_PER_CU;
+		cached = (uint32_t)prop.multiProcessorCount * (uint32_t)per_cu;
+	}
+	*out = cached;
+	return SRF_OK;
+}
+
+static int launch_stream(const srf_loss_args* a, const LossConst& K, ChainScratch S, const float* rays_rgba, const uint32_t* n_rays_counter,
+                         uint32_t* ray_coord_indices, const float* dt, const float* coords, float* compacted_coords, uint32_t* n_compacted_coords_counter,
+                         const void* network_output, void* dloss_doutput, float* loss_output, const float* density_grid_mean, float* rgb_ray_out, hipStream_t st) {
+	const uint32_t n_groups = div_up(a->n_rays, fused::RAYS);
+	fused::Args A;
+	A.K = K;
+	A.n_active = 0;
+	A.rays_rgba = rays_rgba; A.ray_coord_indices = ray_coord_indices; A.dt_arr = dt; A.coords = coords; A.compacted_coords = compacted_coords;
+	A.net = network_output; A.dloss = dloss_doutput; A.loss_output = loss_output; A.rgb_ray_out = rgb_ray_out; A.mean_density = 0.f;
+	const bool hin = a->network_output_dtype == SRF_DTYPE_F16, hout = a->dloss_dtype == SRF_DTYPE_F16;
+	const bool plain = a->rgb_activation == SRF_ACT_NONE && a->density_activation == SRF_ACT_NONE;
+	uint32_t resident = 0;
+	int rc;
+#define SRF_RESIDENT(HI, HO, PL) rc = stream_resident_workgroups<HI, HO, PL>(&resident)
+#define SRF_RESIDENT_IO(PL) do { if (hin && hout) SRF_RESIDENT(true, true, PL); else if (hin) SRF_RESIDENT(true, false, PL); else if (hout) SRF_RESIDENT(false, true, PL); else SRF_RESIDENT(false, false, PL); } while (0)
+	if (plain) SRF_RESIDENT_IO(true); else SRF_RESIDENT_IO(false);
+#undef SRF_RESIDENT_IO
+#undef SRF_RESIDENT
+	if (rc != SRF_OK) return rc;
+	const dim3 grid(n_groups < resident ? n_groups : resident), block(STREAM_THREADS), slow_block(fused::WideGeometry::THREADS), slow_grid(n_groups < 256u ? n_groups : 256u);   // listed groups are few
+	hipLaunchKernelGGL(k_chain_prepare, dim3(div_up(n_groups, PREPARE_WAVES)), dim3(PREPARE_WAVES * WAVE), 0, st, A, n_rays_counter, S, n_groups, (const uint32_t*)n_compacted_coords_counter);
+	hipLaunchKernelGGL(k_chain_items, dim3(div_up(n_groups, ITEMS_THREADS)), dim3(ITEMS_THREADS), 0, st, a->n_rays, n_rays_counter, S);
+	SRF_LAUNCH_CHECK();
+	if (hin) hipLaunchKernelGGL((k_slow_groups<true, false, false>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S);
+	else     hipLaunchKernelGGL((k_slow_groups<false, false, false>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S);
+	SRF_LAUNCH_CHECK();
+#define SRF_STREAM(HI, HO, PL) hipLaunchKernelGGL((k_composite_stream<HI, HO, PL>), grid, block, 0, st, A, n_rays_counter, density_grid_mean, S, n_compacted_coords_counter)
+#define SRF_STREAM_IO(PL) do { if (hin && hout) SRF_STREAM(true, true, PL); else if (hin) SRF_STREAM(true, false, PL); else if (hout) SRF_STREAM(false, true, PL); else SRF_STREAM(false, false, PL); } while (0)
+	if (plain) SRF_STREAM_IO(true); else SRF_STREAM_IO(false);
+#undef SRF_STREAM_IO
+#undef SRF_STREAM
+	SRF_LAUNCH_CHECK();
+#define SRF_SLOW_BWD(HI, HO) hipLaunchKernelGGL((k_slow_groups<HI, HO, true>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S)
+	if (hin && hout) SRF_SLOW_BWD(true, true); else if (hin) SRF_SLOW_BWD(true, false); else if (hout) SRF_SLOW_BWD(false, true); else SRF_SLOW_BWD(false, false);
+#undef SRF_SLOW_BWD
+	SRF_LAUNCH_CHECK();
+#ifdef SRF_STREAM_TIMING
+	{
+		unsigned long long h[36];
+		SRF_HIP(hipStreamSynchronize(st));
+		SRF_HIP(hipMemcpy(h, S.initial + 16, sizeof(h), hipMemcpyDeviceToHost));
+		SRF_HIP(hipMemset(S.initial + 16, 0, sizeof(h)));
+		static const char* names[3][9] = {{"commit", "barrier", "-", "barrier", "chain", "-", "resolve", "count+publish", "-"},
+		                                  {"finish", "barrier", "rest", "barrier", "plan-tail", "rec-wait", "from-records", "part", "-"},
+		                                  {"-", "barrier", "-", "barrier", "wait-loads", "phaseA", "-", "issue-loads", "phaseC"}};
+		for (int role = 0; role < 3; ++role) {
+			const double n = (double)h[role * 12 + 11];
+			if (n == 0) continue;
+			fprintf(stderr, "stream timing, %s (%.0f iterations), mean cycles:", role == 0 ? "ray wave" : role == 1 ? "plan wave" : "sample wave", n);
+			for (int k = 0; k < 9; ++k) fprintf(stderr, " %s %.0f", names[role][k], h[role * 12 + k] / n);
+			fprintf(stderr, "\n");
+		}
+	}
+#endif
+	return SRF_OK;
+}
+
 } // namespace srf
 
 using namespace srf;
@@ -573,6 +773,27 @@ int srf_marcher_create(const srf_marcher_config* cfg, srf_marcher_t** out) {
 	SRF_REQUIRE(cfg->regularization_type == SRF_REG_NONE || cfg->regularization_type == SRF_REG_DISTORTION, "Unknown regularization type.");
 	srf_marcher* m = new srf_marcher();
 	m->cfg = *cfg;
+	// SRF_COMPOSITE_IMPL=unfused (read once, here) selects the three-launch, one-thread-per-ray training compositing for every
+	// call on this marcher; the tests use it to compare the two implementations
+	const char* impl_env = getenv("SRF_COMPOSITE_IMPL");
+	m->force_unfused = impl_env && strcmp(impl_env, "unfused") == 0;
+	// A word of host memory that the device can write: the streaming kernel raises it when its ordered-offset chain gives up, and
+	// the next call reads it without waiting for the device.  Without a device (configuration-only use) there is none.
+	int n_dev = 0;
+	if (hipGetDeviceCount(&n_dev) == hipSuccess && n_dev > 0) {
+		void* host = nullptr;
+		if (hipHostMalloc(&host, 64, hipHostMallocMapped) == hipSuccess) {
+			void* dev = nullptr;
+			if (hipHostGetDevicePointer(&dev, host, 0) == hipSuccess) {
+				m->host_error = (volatile uint32_t*)host;
+				m->host_error_dev = (uint32_t*)dev;
+				*m->host_error = 0u;
+			} else {
+				(void)hipHostFree(host);
+			}
+		}
+		(void)hipGetLastError();
+	}
 	*out = m;
 	return SRF_OK;
 }
@@ -582,6 +803,8 @@ void srf_marcher_destroy(srf_marcher_t* m) {
 	m->ws.release();
 	m->ws2.release();
 	m->reg.release();
+	m->compact_ws.release();
+	if (m->host_error) (void)hipHostFree((void*)m->host_error);
 	delete m;
 }
 
@@ -629,134 +852,23 @@ int srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const 
 		Pcg32 r; r.state = a->rng.state; r.inc = a->rng.inc;
 		K.bg_in[0] = pcg_next_float(r); K.bg_in[1] = pcg_next_float(r); K.bg_in[2] = pcg_next_float(r);
 	}
+	loss_const_background(K);
 	K.color_space = a->color_space;
 	K.train_in_linear = m->cfg.train_in_linear_color;
 	K.thr = m->cfg.transmittance_threshold;
 	K.dt_stride = a->dt_stride;
 
 	const bool hin = a->network_output_dtype == SRF_DTYPE_F16, hout = a->dloss_dtype == SRF_DTYPE_F16;
-	// The distortion regulariser's side buffer is only filled by the three-launch implementation;
-	// SRF_COMPOSITE_IMPL=unfused selects that implementation for everything (for comparisons).
-	// SRF_COMPOSITE_IMPL (read at every call): "lookback" (default) one launch with ordered offsets chained between workgroups;
-	// "twopass" forward pass + scan + backward pass with no waits between workgroups; "unfused" one thread per ray.
-	const char* impl_env = getenv("SRF_COMPOSITE_IMPL");
-	const bool force_unfused = impl_env && strcmp(impl_env, "unfused") == 0;
-	const bool use_twopass = impl_env && strcmp(impl_env, "twopass") == 0;
-	if (m->cfg.regularization_type != SRF_REG_DISTORTION && use_twopass) {
-		const uint32_t n_groups = div_up(a->n_rays, fused::RAYS);
-		const size_t n = a->n_rays;
-		const size_t off_n = 0;
-		const size_t off_cb = align_up(off_n + n * 4, 256);
-		const size_t off_list = align_up(off_cb + n * 4, 256);
-		const size_t off_scan = align_up(off_list + ((size_t)n_groups + 1) * 4, 256);
-		int rc = m->ws2.reserve(off_scan + scan_scratch_bytes(a->n_rays));
+	int rc = check_chain_error(m);
+	if (rc != SRF_OK) return rc;
+	// The distortion regulariser's side buffer is only filled by the three-launch implementation, which also serves a marcher
+	// whose chain has failed before, and one created under SRF_COMPOSITE_IMPL=unfused.
+	if (m->cfg.regularization_type != SRF_REG_DISTORTION && !m->force_unfused && !m->degraded) {
+		rc = m->ws.reserve(chain_layout(a->n_rays).bytes);
 		if (rc != SRF_OK) return rc;
-		char* w = (char*)m->ws2.ptr;
-		uint32_t* n_fwd = (uint32_t*)(w + off_n);
-		uint32_t* cbase = (uint32_t*)(w + off_cb);
-		uint32_t* slow_list = (uint32_t*)(w + off_list);   // [0] = how many groups follow
-		hipLaunchKernelGGL(k_fill_word, dim3(1), dim3(1), 0, st, slow_list, 0u);
-		SRF_LAUNCH_CHECK();
-		fused::Args A;
-		A.K = K;
-		A.n_active = 0;
-		A.rays_rgba = rays_rgba; A.ray_coord_indices = ray_coord_indices; A.dt_arr = dt; A.coords = coords; A.compacted_coords = compacted_coords;
-		A.net = network_output; A.dloss = dloss_doutput; A.loss_output = loss_output; A.rgb_ray_out = nullptr; A.mean_density = 0.f;
-		// enough workgroups to fill the device a few times over; each walks over its share of the groups
-		static int n_cus = 0;
-		if (!n_cus) { hipDeviceProp_t prop; int dev = 0; SRF_HIP(hipGetDevice(&dev)); SRF_HIP(hipGetDeviceProperties(&prop, dev)); n_cus = prop.multiProcessorCount; }
-		uint32_t per_cu = 16;
-		{ const char* v = getenv("SRF_COMPOSITE_BLOCKS_PER_CU"); if (v && atoi(v) >= 1) per_cu = (uint32_t)atoi(v); }
-		const uint32_t blocks = n_groups < (uint32_t)n_cus * per_cu ? n_groups : (uint32_t)n_cus * per_cu;
-		const dim3 grid(blocks), block(fused::THREADS);
-		const dim3 slow_grid(n_groups < 2048u ? n_groups : 2048u);
-		unsigned long long* timing = nullptr;
-#ifdef SRF_FUSED_TIMING
-		static unsigned long long* timing_buf = nullptr;
-		if (!timing_buf) { SRF_HIP(hipMalloc((void**)&timing_buf, 1024 * 64)); SRF_HIP(hipMemset(timing_buf, 0, 1024 * 64)); }
-		timing = timing_buf;
-		auto report = [&](const char* what) {
-			static unsigned long long hs[1024 * 8];
-			unsigned long long h[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-			(void)hipStreamSynchronize(st);
-			(void)hipMemcpy(hs, timing, sizeof(hs), hipMemcpyDeviceToHost);
-			(void)hipMemset(timing, 0, sizeof(hs));
-			for (int i = 0; i < 1024; ++i) for (int k = 0; k < 8; ++k) h[k] += hs[i * 8 + k];
-			if (h[7]) fprintf(stderr, "%s pass, mean cycles per group over %llu iterations: top %.0f  phaseA-compute(+wait) %.0f  plan+issue %.0f  chain+finish %.0f  phaseC %.0f  end %.0f\n",
-			                  what, h[7], (double)h[0] / h[7], (double)h[1] / h[7], (double)h[2] / h[7], (double)h[3] / h[7], (double)h[4] / h[7], (double)h[5] / h[7]);
-		};
-#endif
-#define SRF_PASS(HI, HO, BW) do { \
-		hipLaunchKernelGGL((k_composite_pass<HI, HO, BW>), grid, block, 0, st, A, n_rays_counter, density_grid_mean, n_groups, n_fwd, (const uint32_t*)cbase, slow_list, timing); \
-		hipLaunchKernelGGL((k_composite_pass_slow<HI, HO, BW>), slow_grid, block, 0, st, A, n_rays_counter, density_grid_mean, n_fwd, (const uint32_t*)cbase, (const uint32_t*)slow_list); \
-	} while (0)
-		if (hin) SRF_PASS(true, false, false); else SRF_PASS(false, false, false);
-		SRF_LAUNCH_CHECK();
-#ifdef SRF_FUSED_TIMING
-		report("forward");
-#endif
-		rc = scan_exclusive_u32(n_fwd, cbase, a->n_rays, n_compacted_coords_counter, n_compacted_coords_counter, w + off_scan, st);
-		if (rc != SRF_OK) return rc;
-		A.rgb_ray_out = rgb_ray_out;
-		if (hin && hout) SRF_PASS(true, true, true);
-		else if (hin) SRF_PASS(true, false, true);
-		else if (hout) SRF_PASS(false, true, true);
-		else SRF_PASS(false, false, true);
-#undef SRF_PASS
-		SRF_LAUNCH_CHECK();
-#ifdef SRF_FUSED_TIMING
-		report("backward");
-#endif
-		return SRF_OK;
-	}
-	if (m->cfg.regularization_type != SRF_REG_DISTORTION && !force_unfused) {
-		const uint32_t n_groups = div_up(a->n_rays, fused::RAYS);
-		const size_t off_status = 0;
-		const size_t off_seg = align_up((size_t)n_groups * 8, 256);
-		const size_t off_misc = align_up(off_seg + (size_t)div_up(n_groups, 64) * 8, 256);
-		const void* before = m->ws.ptr;
-		int rc = m->ws.reserve(off_misc + 256 + 1024 * 64);
-		if (rc != SRF_OK) return rc;
-		const bool fresh = m->ws.ptr != before || m->chain_misc_offset != off_misc;
-		m->chain_misc_offset = off_misc;
-		ChainScratch S;
-		S.group_status = (unsigned long long*)((char*)m->ws.ptr + off_status);
-		S.seg_status = (unsigned long long*)((char*)m->ws.ptr + off_seg);
-		S.initial = (uint32_t*)((char*)m->ws.ptr + off_misc) + 1;
-		S.error = S.initial + 1;
-		S.timing = (unsigned long long*)((char*)m->ws.ptr + off_misc + 256);
-		if (fresh) {
-			hipLaunchKernelGGL(k_fill_word, dim3(1), dim3(1), 0, st, S.error, 0u);
-			SRF_LAUNCH_CHECK();
-		}
-		hipLaunchKernelGGL(k_chain_init, dim3(div_up(n_groups, 256)), dim3(256), 0, st, S, n_groups, (const uint32_t*)n_compacted_coords_counter);
-		SRF_LAUNCH_CHECK();
-		fused::Args A;
-		A.K = K;
-		A.n_active = 0;
-		A.rays_rgba = rays_rgba; A.ray_coord_indices = ray_coord_indices; A.dt_arr = dt; A.coords = coords; A.compacted_coords = compacted_coords;
-		A.net = network_output; A.dloss = dloss_doutput; A.loss_output = loss_output; A.rgb_ray_out = rgb_ray_out; A.mean_density = 0.f;
-		const dim3 grid(n_groups), block(fused::THREADS);
-#define SRF_FUSED(HI, HO) hipLaunchKernelGGL((k_composite_fused<HI, HO>), grid, block, 0, st, A, n_rays_counter, density_grid_mean, n_groups, S, n_compacted_coords_counter)
-		if (hin && hout) SRF_FUSED(true, true);
-		else if (hin) SRF_FUSED(true, false);
-		else if (hout) SRF_FUSED(false, true);
-		else SRF_FUSED(false, false);
-#undef SRF_FUSED
-		SRF_LAUNCH_CHECK();
-#ifdef SRF_FUSED_TIMING
-		{
-			static unsigned long long hs[1024 * 8];
-			unsigned long long h[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-			SRF_HIP(hipStreamSynchronize(st));
-			SRF_HIP(hipMemcpy(hs, S.timing, sizeof(hs), hipMemcpyDeviceToHost));
-			SRF_HIP(hipMemset(S.timing, 0, sizeof(hs)));
-			for (int i = 0; i < 1024; ++i) for (int k = 0; k < 8; ++k) h[k] += hs[i * 8 + k];
-			if (h[7] && !fresh) fprintf(stderr, "fused phases, mean cycles per group over %llu groups: setup %.0f  phaseA %.0f  chain %.0f  finish %.0f  lookback %.0f  phaseC %.0f\n",
-			                  h[7], (double)h[0] / h[7], (double)h[1] / h[7], (double)h[2] / h[7], (double)h[3] / h[7], (double)h[4] / h[7], (double)h[5] / h[7]);
-		}
-#endif
-		return SRF_OK;
+		m->chain_error_dev = chain_scratch_at(m->ws.ptr, a->n_rays, nullptr, 0).error;
+		return launch_stream(a, K, chain_scratch_at(m->ws.ptr, a->n_rays, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
+		                     compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, st);
 	}
 
 	const size_t n = a->n_rays;
@@ -764,7 +876,7 @@ int srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const 
 	const size_t off_n = align_up(off_fwd + n * sizeof(FwdRay), 256);
 	const size_t off_cb = align_up(off_n + n * 4, 256);
 	const size_t off_scan = align_up(off_cb + n * 4, 256);
-	int rc = m->ws2.reserve(off_scan + scan_scratch_bytes(a->n_rays));
+	rc = m->ws2.reserve(off_scan + scan_scratch_bytes(a->n_rays));
 	if (rc != SRF_OK) return rc;
 	char* w = (char*)m->ws2.ptr;
 	FwdRay* fwd = (FwdRay*)(w + off_fwd);
@@ -796,10 +908,21 @@ int srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const 
 int srf_marcher_sync_check(srf_marcher_t* m, void* stream) {
 	SRF_REQUIRE(m, "srf_marcher_sync_check: NULL marcher");
 	SRF_HIP(hipStreamSynchronize((hipStream_t)stream));
-	if (!m->ws.ptr || m->chain_misc_offset == (size_t)-1) return SRF_OK;
-	uint32_t flag = 0;
-	SRF_HIP(hipMemcpy(&flag, (char*)m->ws.ptr + m->chain_misc_offset + 8, 4, hipMemcpyDeviceToHost));
-	if (flag) SRF_FAIL(SRF_ERR_HIP, "compositing: a workgroup gave up waiting for its predecessors' sample counts; compacted offsets of the last call are invalid");
+	if (m->chain_error_dev) {
+		uint32_t flag = 0;
+		SRF_HIP(hipMemcpy(&flag, m->chain_error_dev, 4, hipMemcpyDeviceToHost));
+		if (flag && m->host_error) *m->host_error = 1u;
+		if (flag && !m->host_error) {
+			m->degraded = true;
+			SRF_FAIL(SRF_ERR_HIP, "compositing: a workgroup gave up waiting for its predecessors' sample counts; compacted offsets of the last call are invalid");
+		}
+	}
+	return check_chain_error(m);
+}
+
+int srf_marcher_debug_set_lookback_spin_limit(srf_marcher_t* m, uint32_t polls) {
+	SRF_REQUIRE(m, "srf_marcher_debug_set_lookback_spin_limit: NULL marcher");
+	m->lookback_spin_limit = polls;
 	return SRF_OK;
 }
 
@@ -820,20 +943,18 @@ int srf_marcher_volume_rendering(srf_marcher_t* m, const srf_sampler_t* s, const
 	return SRF_OK;
 }
 
-// one process-wide scratch for the orchestrator kernels, which have no object to hang it on
-static srf::Workspace g_compact_ws;
-
-int srf_compact_rays(uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba,
+int srf_compact_rays(srf_marcher_t* m, uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba,
                      srf_ray_payload* dst_payloads, float* dst_rgba, srf_ray_payload* final_payloads, float* final_rgba,
                      uint32_t* n_alive_counter, uint32_t* n_final_counter, void* stream) {
+	SRF_REQUIRE(m, "srf_compact_rays: NULL marcher");
 	if (n == 0) return SRF_OK;
 	SRF_REQUIRE(src_payloads && src_rgba && dst_payloads && dst_rgba && final_payloads && final_rgba && n_alive_counter && n_final_counter,
 	            "srf_compact_rays: NULL buffer");
 	hipStream_t st = (hipStream_t)stream;
 	const size_t stride = align_up((size_t)n * 4, 256);
-	int rc = g_compact_ws.reserve(4 * stride + scan_scratch_bytes(n));
+	int rc = m->compact_ws.reserve(4 * stride + scan_scratch_bytes(n));
 	if (rc != SRF_OK) return rc;
-	char* w = (char*)g_compact_ws.ptr;
+	char* w = (char*)m->compact_ws.ptr;
 	uint32_t* alive = (uint32_t*)w; uint32_t* alive_pos = (uint32_t*)(w + stride);
 	uint32_t* fin = (uint32_t*)(w + 2 * stride); uint32_t* fin_pos = (uint32_t*)(w + 3 * stride);
 	void* scan = w + 4 * stride;

@@ -1,18 +1,20 @@
 // Single-launch training compositing (forward, loss, ordered compaction, backward).
 //
-// One workgroup owns RAYS consecutive rays.  Because a sampler that assigns offsets in ray
+// A group is RAYS consecutive rays.  Because a sampler that assigns offsets in ray
 // order lays the samples of consecutive rays out back to back, the group's samples form
 // one contiguous range, which is streamed through the group in windows of WIN samples:
 //
 //   phase A  (thread <-> sample)  coalesced loads of rgb-sigma and dt; alpha = 1 - exp(-sigma dt);
 //                                 {alpha, colour} of every sample goes to LDS
-//   chain    (lane   <-> ray)     the reference's loop over the ray's samples in order: termination
-//                                 test, weight = alpha * T, colour sum, T *= (1 - alpha); the
-//                                 transmittance after each sample and the colour sum including it
-//                                 replace the sample's LDS record
+//   count    (lane   <-> ray)     the transmittance part of the reference's loop alone (termination test,
+//                                 T *= (1 - alpha)): how many samples the ray consumes.  The group's total
+//                                 is published to the other groups as soon as it is known.
+//   chain    (lane   <-> ray)     the reference's loop over those samples in order: weight = alpha * T,
+//                                 colour sum, T *= (1 - alpha); the transmittance after each sample and
+//                                 the colour sum including it replace the sample's LDS record
 //   finish   (lane   <-> ray)     background, target, loss, gradient of the loss; the group's
 //                                 compacted count is chained to its predecessors' (decoupled
-//                                 look-back over groups in ticket order) to get ordered offsets
+//                                 look-back over groups) to get ordered offsets
 //   phase C  (thread <-> sample)  gradients from the exact per-sample T and colour prefix,
 //                                 stored at the compacted position
 //
@@ -32,16 +34,15 @@
 #include "srf_bodies.h"
 
 #if defined(__HIP_DEVICE_COMPILE__)
+// a value that is the same in every lane of the wave (read from LDS, say), moved to where the compiler knows it is
+#define SRF_UNIFORM_U32(x) ((uint32_t)__builtin_amdgcn_readfirstlane((int)(x)))
 #define SRF_LDS_ADD(p, v) atomicAdd((p), (v))
 #define SRF_LDS_AND(p, v) atomicAnd((p), (v))
 // keeps the instruction scheduler from interleaving the unrolled per-slot bodies, which would
 // multiply the live temporaries by the slot count and cost occupancy
-#ifdef SRF_NO_SLOT_FENCE
-#define SRF_SLOT_FENCE() ((void)0)
-#else
 #define SRF_SLOT_FENCE() __builtin_amdgcn_sched_barrier(0)
-#endif
 #else
+#define SRF_UNIFORM_U32(x) ((uint32_t)(x))
 #define SRF_LDS_ADD(p, v) (*(p) += (v))
 #define SRF_LDS_AND(p, v) (*(p) &= (v))
 #define SRF_SLOT_FENCE() ((void)0)
@@ -50,28 +51,33 @@
 namespace srf {
 namespace fused {
 
-#ifndef SRF_FUSED_RAYS_HI
-#define SRF_FUSED_RAYS_HI 8
-#endif
-#ifndef SRF_FUSED_RAYS_LO
-#define SRF_FUSED_RAYS_LO 8
-#endif
-#ifndef SRF_FUSED_THREADS
-#define SRF_FUSED_THREADS 256
-#endif
-#ifndef SRF_FUSED_WIN
-#define SRF_FUSED_WIN 1792
-#endif
-constexpr uint32_t RAYS_HI = SRF_FUSED_RAYS_HI, RAYS_LO = SRF_FUSED_RAYS_LO;
-constexpr uint32_t RAYS = RAYS_HI * RAYS_LO;   // rays per workgroup (lanes of the first wave that walk a ray during the chain)
-constexpr uint32_t THREADS = SRF_FUSED_THREADS;
-static_assert(RAYS <= 64 && THREADS % 64 == 0 && SRF_FUSED_WIN % SRF_FUSED_THREADS == 0, "group shape");
-constexpr uint32_t WIN = SRF_FUSED_WIN;   // samples per window
-constexpr uint32_t SLOTS = WIN / THREADS;
+constexpr uint32_t RAYS = 64;        // rays per group: one lane of a wavefront per ray during count, chain and finish
+constexpr uint32_t RAYS_HI = 8, RAYS_LO = 8;
+static_assert(RAYS_HI * RAYS_LO == RAYS, "group shape");
+
+// how many threads share the sample-parallel phases of a group and how many samples each of them holds in registers
+// FENCE_SLOTS: keep the scheduler from interleaving the per-slot bodies (a kernel with a tight register budget)
+template <uint32_t THREADS_, uint32_t SLOTS_, bool FENCE_SLOTS_>
+struct Geometry {
+	static constexpr uint32_t THREADS = THREADS_;
+	static constexpr uint32_t SLOTS = SLOTS_;
+	static constexpr uint32_t WIN = THREADS_ * SLOTS_;   // samples per window
+	static constexpr bool FENCE_SLOTS = FENCE_SLOTS_;
+};
+// a whole workgroup of four waves on the samples, windows of 1792: the kernel for groups of any length
+using WideGeometry = Geometry<256, 7, true>;
+// six waves on the samples (two more walk the rays and plan meanwhile), windows of 1920: the streaming kernel
+using StreamGeometry = Geometry<384, 5, false>;
+
 constexpr uint32_t GAP_SLACK = 1024; // a group whose sample range exceeds its sample count by more takes the per-ray path
 constexpr uint32_t CHAIN_UNROLL = 4;
+constexpr uint32_t COUNT_UNROLL = 8;
+constexpr uint32_t NPLAN = 4;        // plans kept at once by a kernel that has three items under way and plans a fourth
 
-enum { M_S0 = 0, M_TOTAL, M_SUM, M_CONTIG, M_N };
+// M_LANE_LO / M_LANE_HI: the rays (lanes) of the group that this plan covers; M_GROUP: which group; M_ITEM: the number
+// of the item that the plan is for (NO_ITEM: none, the plan is a placeholder), set by kernels that number their items
+enum { M_S0 = 0, M_TOTAL, M_SUM, M_CONTIG, M_LANE_LO, M_LANE_HI, M_GROUP, M_ITEM, M_N };
+constexpr uint32_t NO_ITEM = 0xffffffffu;
 
 // per ray, read by phase C
 struct alignas(16) RayOut {
@@ -81,33 +87,101 @@ struct alignas(16) RayOut {
 	uint32_t n_kept;    // samples kept after the compacted-capacity clamp
 };
 
-// where a group's rays lie in the sample buffer; a kernel that prepares the next group while it
-// works on the current one keeps two of these
+// where a group's rays lie in the sample buffer
 struct Plan {
 	uint32_t rabs[RAYS];        // absolute first-sample index per ray
 	uint32_t rbase[RAYS + 1];   // first-sample index relative to the group's first sample
 	uint32_t rn[RAYS];          // samples of the ray on input
 	uint32_t misc[M_N];
 };
+template <class G>
+SRF_HD bool plan_fits_one_window(const Plan& pl) { return pl.misc[M_CONTIG] != 0 && pl.misc[M_TOTAL] <= G::WIN; }
+
+// In how many parts a kernel with windows of G::WIN samples takes a planned group: 1 when it fits one window, 2 when
+// it can be cut at a ray boundary into two stretches that each fit one (rays [0, *split) and [*split, RAYS)), 0 when
+// it cannot (rays not laid out back to back, a single ray longer than a window, more than two windows' worth).
+template <class G>
+SRF_HD uint32_t plan_parts(const Plan& pl, uint32_t* split) {
+	*split = RAYS;
+	if (pl.misc[M_CONTIG] == 0) return 0;
+	const uint32_t total = pl.misc[M_TOTAL];
+	if (total <= G::WIN) return 1;
+	uint32_t s = 0;                                   // the last ray that starts inside the first window
+	for (uint32_t r = 1; r < RAYS; ++r) if (pl.rbase[r] <= G::WIN) s = r;
+	if (s == 0 || total - pl.rbase[s] > G::WIN) return 0;
+	*split = s;
+	return 2;
+}
+
+// The plan of rays [lo, hi) of a planned group, one lane per ray: the other rays own nothing in it.
+SRF_HD void plan_part_lane(uint32_t lane, const Plan& group, uint32_t lo, uint32_t hi, uint32_t g, Plan& part) {
+	const uint32_t start = group.rbase[lo];
+	const uint32_t end = hi < RAYS ? group.rbase[hi] : group.misc[M_TOTAL];
+	const uint32_t total = end - start;
+	const bool mine = lane >= lo && lane < hi;
+	part.rabs[lane] = group.rabs[lane];
+	part.rn[lane] = mine ? group.rn[lane] : 0u;
+	part.rbase[lane] = lane < lo ? 0u : (lane < hi ? group.rbase[lane] - start : total);
+	if (lane == 0) {
+		part.rbase[RAYS] = total;
+		part.misc[M_S0] = group.misc[M_S0] + start;
+		part.misc[M_TOTAL] = total;
+		part.misc[M_SUM] = 0;
+		part.misc[M_CONTIG] = 1;
+		part.misc[M_LANE_LO] = lo;
+		part.misc[M_LANE_HI] = hi;
+		part.misc[M_GROUP] = g;
+	}
+}
+
+// An item is what a streaming workgroup takes at a time: rays [lo, hi) of one group.  A group is one item, or two when
+// it is cut (plan_parts), and the items of all groups, in ray order, are the units of the ordered-offset chain.
+//   x  group
+//   y  lo | hi << 8 | listed << 16   (listed: the streaming path does not take the group, see plan_parts == 0)
+// What k_chain_prepare leaves per group for the pass that numbers the items: items | split << 8 | listed << 16.
+template <class G>
+SRF_HD uint32_t group_items_word(const Plan& pl) {
+	uint32_t split;
+	const uint32_t parts = plan_parts<G>(pl, &split);
+	return (parts == 2 ? 2u : 1u) | (split << 8) | (parts == 0 ? 1u << 16 : 0u);
+}
+SRF_HD uint32_t items_of_group(uint32_t g, uint32_t word, U2 out[2]) {
+	const uint32_t n = word & 0xffu, split = (word >> 8) & 0xffu, listed = word & (1u << 16);
+	out[0].x = g; out[1].x = g;
+	if (n == 2) { out[0].y = 0u | (split << 8); out[1].y = split | (RAYS << 8); }
+	else { out[0].y = (RAYS << 8) | listed; out[1].y = 0; }
+	return n;
+}
+SRF_HD uint32_t item_lo(U2 item) { return item.y & 0xffu; }
+SRF_HD uint32_t item_hi(U2 item) { return (item.y >> 8) & 0xffu; }
+SRF_HD bool item_listed(U2 item) { return (item.y >> 16) != 0; }
 
 constexpr uint32_t NO_OWNER = 0xffu;
 
-struct Shared {
-	Float4 S[WIN];              // phase A: {alpha, r, g, b}; after the chain: {T after the sample, colour prefix r, g, b}
+// one window of samples in LDS
+//   S      phase A: {alpha, r, g, b}; after the chain: {T after the sample, colour prefix r, g, b}
+//   owner  which ray's chain consumed the sample (NO_OWNER: none), written by the chain, read by phase C
+constexpr uint32_t CHAIN_LOOKAHEAD = 8;   // records the ray loops may read past a ray's last sample (they are not used)
+template <class G>
+struct Window {
+	Float4 S[G::WIN + CHAIN_LOOKAHEAD];
+	uint8_t owner[G::WIN];
+};
+
+// per-ray results of a group in LDS
+struct RayLds {
 	RayOut out[RAYS];
-	Plan plan;
-	uint8_t owner[WIN];         // which ray's chain consumed the sample (NO_OWNER: none), written by the chain, read by phase C
 	uint32_t rnf[RAYS];         // samples consumed by the forward pass (early termination)
 	float Tin[RAYS];            // transmittance of the ray at the start of the current window
 	float loss[RAYS];           // loss of the ray, parked until the clamp is known
-	FwdRay fw[RAYS];            // forward results of the per-ray path
+	Float4 carry[RAYS];         // transmittance and colour sum the chain left (for a kernel whose chain and finish run on different waves)
 };
 
-template <bool HALF_IN>
+template <class G, bool HALF_IN>
 struct SlotState {
-	uint32_t raw[SLOTS][HALF_IN ? 2 : 4];
-	float dt[SLOTS];
-	float alpha[SLOTS];
+	uint32_t raw[G::SLOTS][HALF_IN ? 2 : 4];
+	float dt[G::SLOTS];
+	float alpha[G::SLOTS];
 };
 
 struct RayCarry { float T, Cr, Cg, Cb; uint32_t k; uint32_t numsteps; uint32_t done; };
@@ -129,24 +203,12 @@ struct Args {
 
 template <bool HALF_IN>
 SRF_HD void unpack_raw(const uint32_t* raw, float v[4]) {
-	if (HALF_IN) {
+	if constexpr (HALF_IN) {
 		v[0] = half_bits_to_float((uint16_t)(raw[0] & 0xffffu)); v[1] = half_bits_to_float((uint16_t)(raw[0] >> 16));
 		v[2] = half_bits_to_float((uint16_t)(raw[1] & 0xffffu)); v[3] = half_bits_to_float((uint16_t)(raw[1] >> 16));
 	} else {
 		v[0] = srf_u2f(raw[0]); v[1] = srf_u2f(raw[1]); v[2] = srf_u2f(raw[2]); v[3] = srf_u2f(raw[3]);
 	}
-}
-
-// largest r with rbase[r] <= s (rbase is non-decreasing, rbase[0] == 0): two rounds of
-// independent reads (every RAYS_LO-th entry, then the entries inside the chosen run)
-SRF_HD uint32_t ray_of_sample(const Plan& pl, uint32_t s) {
-	uint32_t hi = 0;
-	#pragma unroll
-	for (uint32_t i = 1; i < RAYS_HI; ++i) hi += (pl.rbase[RAYS_LO * i] <= s) ? RAYS_LO : 0u;
-	uint32_t lo = 0;
-	#pragma unroll
-	for (uint32_t i = 1; i < RAYS_LO; ++i) lo += (pl.rbase[hi + i] <= s) ? 1u : 0u;
-	return hi + lo;
 }
 
 // ---- set-up: one lane per ray ------------------------------------------------------------
@@ -191,6 +253,8 @@ SRF_HD void plan_finish_lane(uint32_t lane, uint32_t ray0, const Args& A, Plan& 
 	if (lane == 0) {
 		pl.rbase[RAYS] = total;
 		if ((uint64_t)total > (uint64_t)pl.misc[M_SUM] + GAP_SLACK) pl.misc[M_CONTIG] = 0;
+		pl.misc[M_LANE_LO] = 0; pl.misc[M_LANE_HI] = RAYS;
+		pl.misc[M_GROUP] = ray0 / RAYS;
 	}
 }
 
@@ -201,17 +265,17 @@ SRF_HD void reset_carry(uint32_t lane, const Plan& pl, RayCarry& c) {
 // ---- phase A: thread <-> sample ----------------------------------------------------------
 // loads: every slot inside the group's range is fetched, whether or not a ray owns it (holes left by
 // dropped rays lie between valid samples, inside the buffer), so the loads wait for nothing but the plan
-template <bool HALF_IN>
-SRF_HD void phase_a_load(uint32_t tid, uint32_t win, const Args& A, const Plan& pl, SlotState<HALF_IN>& st) {
+template <class G, bool HALF_IN>
+SRF_HD void phase_a_load(uint32_t tid, uint32_t win, const Args& A, const Plan& pl, SlotState<G, HALF_IN>& st) {
 	const uint32_t total = pl.misc[M_TOTAL], s0 = pl.misc[M_S0];
-	const uint32_t in_window = total - win * WIN < WIN ? total - win * WIN : WIN;
-	const uint32_t n_slots = (in_window + THREADS - 1) / THREADS;     // the same for every thread: unused slot rows are skipped outright
+	const uint32_t in_window = total - win * G::WIN < G::WIN ? total - win * G::WIN : G::WIN;
+	const uint32_t n_slots = (in_window + G::THREADS - 1) / G::THREADS;     // the same for every thread: unused slot rows are skipped outright
 	#pragma unroll
-	for (uint32_t j = 0; j < SLOTS; ++j) {
-		const uint32_t srel = win * WIN + tid + j * THREADS;
+	for (uint32_t j = 0; j < G::SLOTS; ++j) {
+		const uint32_t srel = win * G::WIN + tid + j * G::THREADS;
 		if (j < n_slots && srel < total) {
 			const size_t s = (size_t)s0 + srel;
-			if (HALF_IN) {
+			if constexpr (HALF_IN) {
 				const U2 p = *(const U2*)((const uint32_t*)A.net + s * 2);
 				st.raw[j][0] = p.x; st.raw[j][1] = p.y;
 			} else {
@@ -223,47 +287,151 @@ SRF_HD void phase_a_load(uint32_t tid, uint32_t win, const Args& A, const Plan& 
 	}
 }
 
-// activations and alpha of every slot in the range; {alpha, colour} goes to LDS.  Which ray a sample belongs to
-// does not matter here (a slot in a hole between rays gets a meaningless record that no chain reads); the chain
-// marks the samples it consumes and phase C works from those marks.
-template <bool HALF_IN>
-SRF_HD void phase_a_compute(uint32_t tid, uint32_t win, const Args& A, Shared& sh, const Plan& pl, SlotState<HALF_IN>& st) {
-	const uint32_t total = pl.misc[M_TOTAL];
-	const uint32_t in_window = total - win * WIN < WIN ? total - win * WIN : WIN;
-	const uint32_t n_slots = (in_window + THREADS - 1) / THREADS;
+// The same loads for a plan that fits one window, with the addresses built from one base per array and a 32-bit offset
+// per thread.  A slot past the range re-reads the range's last sample instead of being skipped (its values are not used):
+// nothing here depends on the lane, so the registers need no merging with their old contents.
+template <class G, bool HALF_IN>
+SRF_HD void phase_a_load_single(uint32_t tid, const Args& A, const Plan& pl, SlotState<G, HALF_IN>& st) {
+	const uint32_t total = SRF_UNIFORM_U32(pl.misc[M_TOTAL]), s0 = SRF_UNIFORM_U32(pl.misc[M_S0]);
+	if (total == 0) return;
+	const uint32_t n_slots = (total + G::THREADS - 1) / G::THREADS;
+	const uint32_t* net = (const uint32_t*)A.net + (size_t)s0 * (HALF_IN ? 2 : 4);
+	const float* dt = A.dt_arr + (size_t)s0 * A.K.dt_stride;
 	#pragma unroll
-	for (uint32_t j = 0; j < SLOTS; ++j) {
-		SRF_SLOT_FENCE();
-		const uint32_t q = tid + j * THREADS;
-		const uint32_t srel = win * WIN + q;
-		if (j < n_slots && srel < total) {
-			float v[4];
-			unpack_raw<HALF_IN>(st.raw[j], v);
-			const float density = act_density(v[3], A.K.density_act);
-			const float alpha = 1.f - srf_expf(-density * st.dt[j]);
-			st.alpha[j] = alpha;
-			sh.S[q] = mk4(alpha, act_rgb(v[0], A.K.rgb_act), act_rgb(v[1], A.K.rgb_act), act_rgb(v[2], A.K.rgb_act));
-			sh.owner[q] = (uint8_t)NO_OWNER;
+	for (uint32_t j = 0; j < G::SLOTS; ++j) {
+		if (j < n_slots) {
+			const uint32_t q = tid + j * G::THREADS;
+			const uint32_t srel = q < total ? q : total - 1;
+			if constexpr (HALF_IN) {
+				const U2 p = *(const U2*)(net + srel * 2u);
+				st.raw[j][0] = p.x; st.raw[j][1] = p.y;
+			} else {
+				const U4 p = *(const U4*)(net + srel * 4u);
+				st.raw[j][0] = p.x; st.raw[j][1] = p.y; st.raw[j][2] = p.z; st.raw[j][3] = p.w;
+			}
+			st.dt[j] = dt[(size_t)srel * A.K.dt_stride];
 		}
 	}
 }
 
-template <bool HALF_IN>
-SRF_HD void phase_a(uint32_t tid, uint32_t win, const Args& A, Shared& sh, const Plan& pl, SlotState<HALF_IN>& st) {
-	phase_a_load<HALF_IN>(tid, win, A, pl, st);
-	phase_a_compute<HALF_IN>(tid, win, A, sh, pl, st);
+// activations and alpha of every slot in the range; {alpha, colour} goes to LDS.  Which ray a sample belongs to
+// does not matter here (a slot in a hole between rays gets a meaningless record that no chain reads); the chain
+// marks the samples it consumes and phase C works from those marks.
+// PLAIN: both activations are "None", known at compile time (the arithmetic is the same, the switches are gone)
+template <class G, bool HALF_IN, bool PLAIN = false>
+SRF_HD void phase_a_compute(uint32_t tid, uint32_t win, const Args& A, Window<G>& w, const Plan& pl, SlotState<G, HALF_IN>& st) {
+	const int rgb_act = PLAIN ? (int)SRF_ACT_NONE : A.K.rgb_act, density_act = PLAIN ? (int)SRF_ACT_NONE : A.K.density_act;
+	const uint32_t total = pl.misc[M_TOTAL];
+	const uint32_t in_window = total - win * G::WIN < G::WIN ? total - win * G::WIN : G::WIN;
+	const uint32_t n_slots = (in_window + G::THREADS - 1) / G::THREADS;
+	#pragma unroll
+	for (uint32_t j = 0; j < G::SLOTS; ++j) {
+		if (G::FENCE_SLOTS) SRF_SLOT_FENCE();
+		const uint32_t q = tid + j * G::THREADS;
+		const uint32_t srel = win * G::WIN + q;
+		if (j < n_slots && srel < total) {
+			float v[4];
+			unpack_raw<HALF_IN>(st.raw[j], v);
+			const float density = act_density(v[3], density_act);
+			const float alpha = 1.f - srf_expf(-density * st.dt[j]);
+			st.alpha[j] = alpha;
+			w.S[q] = mk4(alpha, act_rgb(v[0], rgb_act), act_rgb(v[1], rgb_act), act_rgb(v[2], rgb_act));
+			w.owner[q] = (uint8_t)NO_OWNER;
+		}
+	}
 }
 
-// ---- chain: lane <-> ray (ray_marcher.cu:63-79; the same loop again at :171-182) ---------
+template <class G, bool HALF_IN, bool PLAIN = false>
+SRF_HD void phase_a(uint32_t tid, uint32_t win, const Args& A, Window<G>& w, const Plan& pl, SlotState<G, HALF_IN>& st) {
+	phase_a_load<G, HALF_IN>(tid, win, A, pl, st);
+	phase_a_compute<G, HALF_IN, PLAIN>(tid, win, A, w, pl, st);
+}
+
+// ---- count: lane <-> ray (the transmittance half of ray_marcher.cu:63-79) -------------------
+// How many samples the reference's loop consumes before the transmittance falls below the threshold: the same
+// T *= (1 - alpha) sequence the chain runs, without the colours.  For groups that fit one window.
+// Every lane runs n_max steps (the largest count among the lanes that run together) without branching: a lane keeps
+// multiplying after its ray has ended or terminated, which changes nothing, and latches the first step at which the
+// reference's test `T < threshold` (made before a sample is consumed) holds.  Reads past the ray's end are clamped to the
+// window's padding.
+template <class G>
+SRF_HD uint32_t count_lane(uint32_t lane, uint32_t n_max, const Args& A, const Window<G>& w, const Plan& pl) {
+	const Float4* S = w.S;
+	const uint32_t last = G::WIN + CHAIN_LOOKAHEAD - 1;
+	const uint32_t base = pl.rbase[lane];
+	uint32_t cnt = pl.rn[lane];
+	float T = 1.f;
+	const float thr = A.K.thr;
+	for (uint32_t k = 0; k < n_max; k += COUNT_UNROLL) {
+		float a[COUNT_UNROLL];
+		#pragma unroll
+		for (uint32_t u = 0; u < COUNT_UNROLL; ++u) a[u] = S[base + k + u < last ? base + k + u : last].x;
+		#pragma unroll
+		for (uint32_t u = 0; u < COUNT_UNROLL; ++u) {
+			cnt = (T < thr && k + u < cnt) ? k + u : cnt;
+			T *= (1.f - a[u]);
+		}
+	}
+	return cnt;
+}
+
+// ---- chain with the count known: lane <-> ray (ray_marcher.cu:63-79, :171-182) -------------------
+// The reference's loop over the n_fwd samples count_lane found: no termination test is left in it.  Every lane runs
+// n_max steps (the largest n_fwd among the lanes that run together); steps past a lane's n_fwd change nothing.
+// The steps [k_lo, k_hi) of that loop (k_lo a multiple of CHAIN_UNROLL; the lane's ray is carried in c from one stretch to the next).
+template <class G>
+SRF_HD void chain_counted_steps(uint32_t lane, uint32_t n_fwd, uint32_t k_lo, uint32_t k_hi, Window<G>& w, const Plan& pl, RayCarry& c) {
+	const uint32_t base = pl.rbase[lane];
+	float T = c.T, r = c.Cr, g = c.Cg, b = c.Cb;
+	for (uint32_t k = k_lo; k < k_hi; k += CHAIN_UNROLL) {
+		Float4 v[CHAIN_UNROLL];
+		#pragma unroll
+		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) v[u] = w.S[base + k + u < G::WIN + CHAIN_LOOKAHEAD - 1 ? base + k + u : G::WIN + CHAIN_LOOKAHEAD - 1];
+		#pragma unroll
+		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) {
+			if (k + u < n_fwd) {
+				const float alpha = v[u].x;
+				const float weight = alpha * T;
+				r += weight * v[u].y; g += weight * v[u].z; b += weight * v[u].w;
+				T *= (1.f - alpha);
+				w.S[base + k + u] = mk4(T, r, g, b);
+				w.owner[base + k + u] = (uint8_t)lane;
+			}
+		}
+	}
+	c.T = T; c.Cr = r; c.Cg = g; c.Cb = b;
+}
+SRF_HD void chain_counted_begin(RayCarry& c) { c.T = 1.f; c.Cr = 0.f; c.Cg = 0.f; c.Cb = 0.f; }
+SRF_HD void chain_counted_end(uint32_t lane, uint32_t n_fwd, RayLds& rl, const Plan& pl, RayCarry& c) {
+	c.k = n_fwd; c.numsteps = pl.rn[lane]; c.done = 0;
+	rl.rnf[lane] = n_fwd;
+	rl.carry[lane] = mk4(c.T, c.Cr, c.Cg, c.Cb);
+}
+template <class G>
+SRF_HD void chain_counted(uint32_t lane, uint32_t n_fwd, uint32_t n_max, Window<G>& w, RayLds& rl, const Plan& pl, RayCarry& c) {
+	chain_counted_begin(c);
+	chain_counted_steps<G>(lane, n_fwd, 0, n_max, w, pl, c);
+	chain_counted_end(lane, n_fwd, rl, pl, c);
+}
+
+// where chain_counted left the lane's ray, read back by another wave
+SRF_HD void carry_from_lds(uint32_t lane, const RayLds& rl, const Plan& pl, RayCarry& c) {
+	const Float4 v = rl.carry[lane];
+	c.T = v.x; c.Cr = v.y; c.Cg = v.z; c.Cb = v.w;
+	c.k = rl.rnf[lane]; c.numsteps = pl.rn[lane]; c.done = 0;
+}
+
+// ---- chain over one window of a longer group: lane <-> ray (ray_marcher.cu:63-79; the same loop again at :171-182) ----
 // Walks the ray's samples inside this window in order: early-termination test, weight,
 // colour sum, transmittance; leaves {T after the sample, colour sum including it} in place.
-SRF_HD void chain(uint32_t lane, uint32_t win, const Args& A, Shared& sh, const Plan& pl, RayCarry& c) {
-	sh.Tin[lane] = c.T;
+template <class G>
+SRF_HD void chain(uint32_t lane, uint32_t win, const Args& A, Window<G>& w, RayLds& rl, const Plan& pl, RayCarry& c) {
+	rl.Tin[lane] = c.T;
 	const uint32_t base = pl.rbase[lane];
-	const uint32_t win_lo = win * WIN;
+	const uint32_t win_lo = win * G::WIN;
 	// samples of this ray that lie in the window: k in [c.k, k_end)
 	uint32_t k_end = c.numsteps;
-	if (base + k_end > win_lo + WIN) k_end = win_lo + WIN > base ? win_lo + WIN - base : 0;
+	if (base + k_end > win_lo + G::WIN) k_end = win_lo + G::WIN > base ? win_lo + G::WIN - base : 0;
 	float T = c.T, r = c.Cr, g = c.Cg, b = c.Cb;
 	uint32_t k = c.k;
 	bool stop = c.done != 0;     // a ray that terminated in an earlier window stays where it stopped
@@ -272,7 +440,7 @@ SRF_HD void chain(uint32_t lane, uint32_t win, const Args& A, Shared& sh, const 
 		#pragma unroll
 		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) {
 			const uint32_t kk = k + u < k_end ? k + u : k_end - 1;     // clamped: stays inside the ray
-			v[u] = sh.S[base + kk - win_lo];
+			v[u] = w.S[base + kk - win_lo];
 		}
 		#pragma unroll
 		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) {
@@ -282,101 +450,159 @@ SRF_HD void chain(uint32_t lane, uint32_t win, const Args& A, Shared& sh, const 
 			const float weight = alpha * T;
 			r += weight * v[u].y; g += weight * v[u].z; b += weight * v[u].w;
 			T *= (1.f - alpha);
-			sh.S[base + k - win_lo] = mk4(T, r, g, b);
-			sh.owner[base + k - win_lo] = (uint8_t)lane;
+			w.S[base + k - win_lo] = mk4(T, r, g, b);
+			w.owner[base + k - win_lo] = (uint8_t)lane;
 			++k;
 		}
 	}
 	c.T = T; c.Cr = r; c.Cg = g; c.Cb = b;
 	c.k = k;
 	c.done = stop ? 1u : 0u;
-	sh.rnf[lane] = k;
+	rl.rnf[lane] = k;
 }
 
 // ---- finish: lane <-> ray (ray_marcher.cu:81-109, 128-133) -------------------------------
-SRF_HD void finish_ray(uint32_t lane, uint32_t ray0, const Args& A, Shared& sh, RayCarry& c, Float4 target_rgba) {
+SRF_HD void finish_ray(uint32_t lane, uint32_t ray0, const Args& A, RayLds& rl, RayCarry& c, Float4 target_rgba, uint32_t lane_lo = 0, uint32_t lane_hi = RAYS) {
 	const uint32_t i = ray0 + lane;
-	if (i >= A.n_active) { sh.rnf[lane] = 0; return; }
+	if (i >= A.n_active || lane < lane_lo || lane >= lane_hi) { rl.rnf[lane] = 0; return; }
 	float target[3], bg[3];
 	target_and_background(A.K, target_rgba, target, bg);
 	float r = c.Cr, g = c.Cg, b = c.Cb;
 	if (c.k == c.numsteps) { r += c.T * bg[0]; g += c.T * bg[1]; b += c.T * bg[2]; }
-	RayOut& o = sh.out[lane];
+	RayOut& o = rl.out[lane];
 	o.c[0] = r; o.c[1] = g; o.c[2] = b;
 	float lo[3];
 	loss_channel(A.K.loss_type, target[0], r, &lo[0], &o.g[0]);
 	loss_channel(A.K.loss_type, target[1], g, &lo[1], &o.g[1]);
 	loss_channel(A.K.loss_type, target[2], b, &lo[2], &o.g[2]);
-	sh.loss[lane] = (((lo[0] + lo[1]) + lo[2]) / 3.0f) / (float)A.K.n_rays;
-	sh.rnf[lane] = c.k;
+	rl.loss[lane] = (((lo[0] + lo[1]) + lo[2]) / 3.0f) / (float)A.K.n_rays;
+	rl.rnf[lane] = c.k;
 	if (A.rgb_ray_out) { A.rgb_ray_out[3 * (size_t)i] = r; A.rgb_ray_out[3 * (size_t)i + 1] = g; A.rgb_ray_out[3 * (size_t)i + 2] = b; }
 }
 
 // after the ordered offset of the ray is known (ray_marcher.cu:116-131)
-SRF_HD void commit_ray(uint32_t lane, uint32_t ray0, uint32_t cbase, const Args& A, Shared& sh) {
+// write_loss = false: the ray's loss is written later, by commit_loss (a kernel whose finish may still be running on another wave)
+SRF_HD void commit_ray(uint32_t lane, uint32_t ray0, uint32_t cbase, const Args& A, RayLds& rl, uint32_t lane_lo = 0, uint32_t lane_hi = RAYS, bool write_loss = true) {
 	const uint32_t i = ray0 + lane;
-	RayOut& o = sh.out[lane];
+	RayOut& o = rl.out[lane];
 	o.cbase = cbase;
-	if (i >= A.n_active) { o.n_kept = 0; return; }
-	uint32_t n = sh.rnf[lane];
+	if (i >= A.n_active || lane < lane_lo || lane >= lane_hi) { o.n_kept = 0; return; }
+	uint32_t n = rl.rnf[lane];
 	const uint32_t room = A.K.n_max_compacted - (A.K.n_max_compacted < cbase ? A.K.n_max_compacted : cbase);
 	n = room < n ? room : n;
 	o.n_kept = n;
 	A.ray_coord_indices[2 * (size_t)i] = n;
 	A.ray_coord_indices[2 * (size_t)i + 1] = cbase;
-	if (n != 0 && A.loss_output) A.loss_output[i] = sh.loss[lane];
+	if (write_loss && n != 0 && A.loss_output) A.loss_output[i] = rl.loss[lane];
+}
+
+SRF_HD void commit_loss(uint32_t lane, uint32_t ray0, const Args& A, const RayLds& rl, uint32_t lane_lo = 0, uint32_t lane_hi = RAYS) {
+	const uint32_t i = ray0 + lane;
+	if (i >= A.n_active || lane < lane_lo || lane >= lane_hi) return;
+	if (rl.out[lane].n_kept != 0 && A.loss_output) A.loss_output[i] = rl.loss[lane];
 }
 
 // ---- phase C: thread <-> sample (ray_marcher.cu:171-201) ---------------------------------
-template <bool HALF_IN, bool HALF_OUT>
-SRF_HD void phase_c(uint32_t tid, uint32_t win, const Args& A, Shared& sh, const Plan& pl, SlotState<HALF_IN>& st) {
-	const float l2_reg = A.K.rgb_act == SRF_ACT_EXPONENTIAL ? 1e-4f : 0.0f;
+// COPY_COORDS = false: the kept samples' coordinates are moved elsewhere (coords_copy_single)
+template <class G, bool HALF_IN, bool HALF_OUT, bool PLAIN = false, bool COPY_COORDS = true>
+SRF_HD void phase_c(uint32_t tid, uint32_t win, const Args& A, const Window<G>& w, const RayLds& rl, const Plan& pl, SlotState<G, HALF_IN>& st) {
+	const int rgb_act = PLAIN ? (int)SRF_ACT_NONE : A.K.rgb_act, density_act = PLAIN ? (int)SRF_ACT_NONE : A.K.density_act;
+	const float l2_reg = rgb_act == SRF_ACT_EXPONENTIAL ? 1e-4f : 0.0f;
 	const float l1_reg_density = (A.K.use_grid && (A.mean_density < A.K.min_optical_thickness)) ? 1e-4f : 0.0f;
 	const uint32_t total = pl.misc[M_TOTAL];
-	const uint32_t in_window = total - win * WIN < WIN ? total - win * WIN : WIN;
-	const uint32_t n_slots = (in_window + THREADS - 1) / THREADS;
+	const uint32_t in_window = total - win * G::WIN < G::WIN ? total - win * G::WIN : G::WIN;
+	const uint32_t n_slots = (in_window + G::THREADS - 1) / G::THREADS;
 	#pragma unroll
-	for (uint32_t j = 0; j < SLOTS; ++j) {
-		SRF_SLOT_FENCE();
+	for (uint32_t j = 0; j < G::SLOTS; ++j) {
+		if (G::FENCE_SLOTS) SRF_SLOT_FENCE();
 		if (j >= n_slots) continue;
-		const uint32_t q = tid + j * THREADS;
-		if (win * WIN + q >= total) continue;
-		const uint32_t r = sh.owner[q];
+		const uint32_t q = tid + j * G::THREADS;
+		if (win * G::WIN + q >= total) continue;
+		const uint32_t r = w.owner[q];
 		if (r >= RAYS) continue;
-		const uint32_t k = win * WIN + q - pl.rbase[r];
-		const Float4 og = *(const Float4*)&sh.out[r].g[0];      // g.xyz, cbase
-		const Float4 oc = *(const Float4*)&sh.out[r].c[0];      // c.xyz, n_kept
+		const uint32_t k = win * G::WIN + q - pl.rbase[r];
+		const Float4 og = *(const Float4*)&rl.out[r].g[0];      // g.xyz, cbase
+		const Float4 oc = *(const Float4*)&rl.out[r].c[0];      // c.xyz, n_kept
 		if (k >= srf_f2u(oc.w)) continue;
-		const Float4 after = sh.S[q];                            // T after the sample, colour prefix including it
-		const float T_before = (k == 0) ? 1.f : (q == 0 ? sh.Tin[r] : sh.S[q - 1].x);
+		const Float4 after = w.S[q];                             // T after the sample, colour prefix including it
+		const float T_before = (k == 0) ? 1.f : (q == 0 ? rl.Tin[r] : w.S[q - 1].x);
 		float v[4];
 		unpack_raw<HALF_IN>(st.raw[j], v);
-		const float cr = act_rgb(v[0], A.K.rgb_act), cg = act_rgb(v[1], A.K.rgb_act), cb = act_rgb(v[2], A.K.rgb_act);
+		const float cr = act_rgb(v[0], rgb_act), cg = act_rgb(v[1], rgb_act), cb = act_rgb(v[2], rgb_act);
 		const float weight = st.alpha[j] * T_before;
 		const float T = after.x;
-		const float d0 = A.K.loss_scale * ((weight * og.x) * act_rgb_derivative(v[0], A.K.rgb_act) + srf_max(0.0f, l2_reg * v[0]));
-		const float d1 = A.K.loss_scale * ((weight * og.y) * act_rgb_derivative(v[1], A.K.rgb_act) + srf_max(0.0f, l2_reg * v[1]));
-		const float d2 = A.K.loss_scale * ((weight * og.z) * act_rgb_derivative(v[2], A.K.rgb_act) + srf_max(0.0f, l2_reg * v[2]));
+		const float d0 = A.K.loss_scale * ((weight * og.x) * act_rgb_derivative(v[0], rgb_act) + srf_max(0.0f, l2_reg * v[0]));
+		const float d1 = A.K.loss_scale * ((weight * og.y) * act_rgb_derivative(v[1], rgb_act) + srf_max(0.0f, l2_reg * v[1]));
+		const float d2 = A.K.loss_scale * ((weight * og.z) * act_rgb_derivative(v[2], rgb_act) + srf_max(0.0f, l2_reg * v[2]));
 		const float sx = oc.x - after.y, sy = oc.y - after.z, sz = oc.z - after.w;
-		const float dd = act_density_derivative(v[3], A.K.density_act);
+		const float dd = act_density_derivative(v[3], density_act);
 		const float dotv = (og.x * (T * cr - sx) + og.y * (T * cg - sy)) + og.z * (T * cb - sz);
 		const float dmlp = dd * (st.dt[j] * dotv);
 		const float d3 = A.K.loss_scale * dmlp + (v[3] < 0 ? -l1_reg_density : 0.0f);
 		const size_t o = (size_t)srf_f2u(og.w) + k;
+		// One vector store per sample when the records are 4 wide (the reference's padded_output_width).  The general
+		// case goes through volatile pointers only to keep the compiler from folding both cases into scalar stores.
 		if (HALF_OUT) {
-			uint16_t* p = (uint16_t*)A.dloss + o * A.K.out_width;
-			p[0] = float_to_half_bits(d0); p[1] = float_to_half_bits(d1); p[2] = float_to_half_bits(d2); p[3] = float_to_half_bits(d3);
-		} else if ((A.K.out_width & 3u) == 0) {
-			*(Float4*)((float*)A.dloss + o * A.K.out_width) = mk4(d0, d1, d2, d3);
+			const uint32_t lo = (uint32_t)float_to_half_bits(d0) | ((uint32_t)float_to_half_bits(d1) << 16);
+			const uint32_t hi = (uint32_t)float_to_half_bits(d2) | ((uint32_t)float_to_half_bits(d3) << 16);
+			if (A.K.out_width == 4) {
+				U2 v; v.x = lo; v.y = hi;
+				*((U2*)A.dloss + o) = v;
+			} else {
+				volatile uint16_t* p = (volatile uint16_t*)A.dloss + o * A.K.out_width;
+				p[0] = (uint16_t)(lo & 0xffffu); p[1] = (uint16_t)(lo >> 16); p[2] = (uint16_t)(hi & 0xffffu); p[3] = (uint16_t)(hi >> 16);
+			}
+		} else if (A.K.out_width == 4) {
+			*((Float4*)A.dloss + o) = mk4(d0, d1, d2, d3);
 		} else {
-			float* p = (float*)A.dloss + o * A.K.out_width;
+			volatile float* p = (volatile float*)A.dloss + o * A.K.out_width;
 			p[0] = d0; p[1] = d1; p[2] = d2; p[3] = d3;
 		}
-		if (A.compacted_coords) {
-			const size_t s = (size_t)pl.misc[M_S0] + (size_t)win * WIN + q;
-			for (int c = 0; c < 7; ++c) A.compacted_coords[7 * o + c] = A.coords[7 * s + c];
+		if (COPY_COORDS && A.compacted_coords) {
+			const size_t s = (size_t)pl.misc[M_S0] + (size_t)win * G::WIN + q;
+			float cc[7];
+			for (int c = 0; c < 7; ++c) cc[c] = A.coords[7 * s + c];
+			for (int c = 0; c < 7; ++c) A.compacted_coords[7 * o + c] = cc[c];
 		}
 	}
+}
+
+// ---- coordinates of the kept samples of a one-window plan: lane <-> sample (ray_marcher.cu:196-199) ----
+// By the 64 lanes of one wave, COORDS_DEPTH rows of 64 samples at a time so that several rows' loads are under way together.
+constexpr uint32_t COORDS_DEPTH = 8;
+template <class G>
+SRF_HD void coords_copy_rows(uint32_t lane, uint32_t q0, const Args& A, const Window<G>& w, const RayLds& rl, const Plan& pl) {
+	const uint32_t total = pl.misc[M_TOTAL];
+	const float* src = A.coords + 7 * (size_t)pl.misc[M_S0];
+	float cc[COORDS_DEPTH][7];
+	size_t o[COORDS_DEPTH];
+	bool ok[COORDS_DEPTH];
+	#pragma unroll
+	for (uint32_t u = 0; u < COORDS_DEPTH; ++u) {
+		const uint32_t q = q0 + u * RAYS + lane;
+		ok[u] = false; o[u] = 0;
+		if (q < total) {
+			const uint32_t r = w.owner[q];
+			if (r < RAYS) {
+				const uint32_t k = q - pl.rbase[r];
+				if (k < rl.out[r].n_kept) {
+					ok[u] = true;
+					o[u] = (size_t)rl.out[r].cbase + k;
+					for (int c = 0; c < 7; ++c) cc[u][c] = src[7 * q + c];
+				}
+			}
+		}
+	}
+	#pragma unroll
+	for (uint32_t u = 0; u < COORDS_DEPTH; ++u) {
+		if (ok[u]) for (int c = 0; c < 7; ++c) A.compacted_coords[7 * o[u] + c] = cc[u][c];
+	}
+}
+template <class G>
+SRF_HD void coords_copy_single(uint32_t lane, const Args& A, const Window<G>& w, const RayLds& rl, const Plan& pl) {
+	if (!A.compacted_coords) return;
+	const uint32_t total = SRF_UNIFORM_U32(pl.misc[M_TOTAL]);
+	for (uint32_t q0 = 0; q0 < total; q0 += COORDS_DEPTH * RAYS) coords_copy_rows<G>(lane, q0, A, w, rl, pl);
 }
 
 } // namespace fused

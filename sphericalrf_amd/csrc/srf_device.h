@@ -85,6 +85,9 @@ SRF_HD float half_bits_to_float(uint16_t h) {
 
 SRF_HD uint16_t float_to_half_bits(float f) {
 #if defined(__HIP_DEVICE_COMPILE__)
+	// The value converted is the binary32 result already rounded: without this the compiler may merge the multiplication that
+	// produced it with the conversion into one mixed-precision instruction that rounds once, which is not what the host does.
+	asm volatile("" : "+v"(f));
 	const _Float16 v = (_Float16)f;   // round to nearest even
 	uint16_t h;
 	__builtin_memcpy(&h, &v, 2);

@@ -58,8 +58,14 @@ struct srf_sampler {
 
 struct srf_marcher {
 	srf_marcher_config cfg;
-	srf::Workspace ws;
-	srf::Workspace ws2;   // per-ray forward results of the three-launch compositing
-	srf::Workspace reg;   // reg_distortion_buffer (ray_marcher.h:79-80)
-	size_t chain_misc_offset = (size_t)-1;
+	srf::Workspace ws;          // ordered-offset chain of the streaming compositing kernel
+	srf::Workspace ws2;         // per-ray forward results of the three-launch compositing
+	srf::Workspace reg;         // reg_distortion_buffer (ray_marcher.h:79-80)
+	srf::Workspace compact_ws;  // flags and positions of srf_marcher_compact_rays
+	bool force_unfused = false;             // SRF_COMPOSITE_IMPL=unfused at creation
+	bool degraded = false;                  // the chain has failed once: every later call uses the three-launch implementation
+	volatile uint32_t* host_error = nullptr; // host word the streaming kernel raises when its chain gives up (pinned, device-writable)
+	uint32_t* host_error_dev = nullptr;      // the same word as the device addresses it
+	uint32_t* chain_error_dev = nullptr;     // device word of the last streaming launch (NULL before the first)
+	uint32_t lookback_spin_limit = 1u << 22; // polls before a group gives up waiting for its predecessors
 };

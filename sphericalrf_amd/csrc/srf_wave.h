@@ -26,6 +26,12 @@ __device__ inline uint32_t wave_sum_u32(uint32_t v) {
 	return v;
 }
 
+__device__ inline uint32_t wave_max_u32(uint32_t v) {
+	#pragma unroll
+	for (uint32_t d = WAVE / 2; d > 0; d >>= 1) { const uint32_t o = (uint32_t)__shfl_xor((int)v, d, WAVE); v = o > v ? o : v; }
+	return v;
+}
+
 // sum over a workgroup of THREADS threads (multiple of 64); lds holds THREADS/64 words.
 // Every thread receives the total.
 template <uint32_t THREADS>

@@ -206,3 +206,63 @@ def workload(config_id, scale=1.0):
                     blobs=dict(n_blobs=48, max_radius=0.3, sigma_range=(0.04, 0.08), seed=46, n_satellites=16, satellite_sigma=0.09),
                     occupancy=("level", 0.3), shell=(0.9, 1.0, 0.66), seed=46)
     raise ValueError("config_id must be 1..5")
+
+
+# ---- workload files for the native (torch-free) step driver -------------------------------------
+def sampler_config_struct(cfg):
+    """the "samlper" dict as the C struct srf_sampler_config (include/srf_hip.h), through the same mapping api.OccupancySampler uses"""
+    from . import api
+    return api.sampler_config_from_dict(cfg)
+
+
+def write_workload_file(path, config_id, bitfield, scale=1.0, table_rows=1 << 16):
+    """Writes what tests/cpp/step_bench.cpp reads: magic, srf_sampler_config, cameras, image size and focal length, the occupancy
+    bitfield (numpy uint8, cascade-major) and a (table_rows, 4) table of (r, g, b, sigma) rows."""
+    import ctypes
+    import struct
+    w = workload(config_id, scale)
+    c = sampler_config_struct(w["sampler"])
+    raw = bytes(ctypes.string_at(ctypes.addressof(c), ctypes.sizeof(c)))
+    cams = np.ascontiguousarray(w["cameras"], np.float32)
+    bits = np.ascontiguousarray(bitfield, np.uint8)
+    table = field_table(table_rows, 50 + config_id)
+    with open(path, "wb") as f:
+        f.write(b"SRFWLD01")
+        f.write(struct.pack("<I", len(raw)))
+        f.write(raw)
+        f.write(struct.pack("<Iiiff", cams.shape[0], int(w["resolution"][0]), int(w["resolution"][1]), float(w["focal"][0]), float(w["focal"][1])))
+        f.write(cams.tobytes())
+        f.write(struct.pack("<I", bits.size))
+        f.write(bits.tobytes())
+        f.write(struct.pack("<I", table.shape[0]))
+        f.write(table.tobytes())
+    return path
+
+
+def _main():
+    """python -m sphericalrf_amd.scene --config 4 --out FILE: builds the workload's grid on the GPU, lets the HIP library turn it
+    into the bitfield, and writes the workload file."""
+    import argparse
+    import torch
+    from . import api
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--config", type=int, default=4)
+    ap.add_argument("--scale", type=float, default=1.0)
+    ap.add_argument("--out", required=True)
+    a = ap.parse_args()
+    w = workload(a.config, a.scale)
+    centres, sigmas = blob_set(**w["blobs"])
+    gs = w["sampler"]["grid_size"]
+    gs = (gs,) * 3 if isinstance(gs, int) else gs
+    grid = density_grid_from_blobs(gs, w["sampler"]["num_cascades"], centres, sigmas, w["occupancy"], w["shell"], w["seed"], device="cuda")
+    s = api.OccupancySampler(w["sampler"])
+    s.set_density_grid(grid)
+    s.update_grid_bitfield()
+    torch.cuda.synchronize()
+    bits = s.density_grid_bitfield.cpu().numpy()
+    write_workload_file(a.out, a.config, bits, a.scale)
+    print("%s: config %d, %d bitfield bytes, %.4f of bits set" % (a.out, a.config, bits.size, float(np.unpackbits(bits).mean())))
+
+
+if __name__ == "__main__":
+    _main()

@@ -9,6 +9,7 @@ static uint64_t g_radius_hist[8][4] = {};   // [cascade][radius 0, 1-block, 2-3,
 #define SRF_COUNT_RADIUS(n, level) (++g_radius_hist[(level) & 7][(n) == 0 ? 0 : ((n) >> (level)) <= 1 ? 1 : ((n) >> (level)) <= 3 ? 2 : 3])
 #include <cstring>
 #include <vector>
+#include <cstdlib>
 #include <algorithm>
 #include "../../sphericalrf_amd/csrc/srf_bodies.h"
 #include "../../sphericalrf_amd/csrc/srf_composite_fused.h"
@@ -37,156 +38,145 @@ static LossConst make_loss_const(const orc_loss_args* a) {
 		Pcg32 r; r.state = a->rng.state; r.inc = a->rng.inc;
 		K.bg_in[0] = pcg_next_float(r); K.bg_in[1] = pcg_next_float(r); K.bg_in[2] = pcg_next_float(r);
 	}
+	loss_const_background(K);
 	K.color_space = a->color_space; K.train_in_linear = a->train_in_linear_color; K.thr = a->transmittance_threshold; K.dt_stride = a->dt_stride;
 	return K;
 }
 
 
-// The single-launch compositing kernel, group by group and phase by phase, in the kernel's control flow.
+// The single-launch compositing, group by group and phase by phase, in the control flow of the device kernels: the
+// groups the streaming kernel does not take (rays not laid out back to back, more samples than one window) get their
+// forward pass first and leave their per-ray counts; the streaming loop then runs every group in order (count, chain
+// with the count known, finish, ordered offsets, phase C), handing the listed groups only their offsets; the listed
+// groups' second forward pass and their gradients come last.
 template <bool HI, bool HO>
 static void run_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n_rays_counter, uint32_t* ray_coord_indices, const float* dt,
                       const float* coords, float* compacted_coords, uint32_t* n_compacted_counter, const void* net, void* dloss, float* loss_output,
                       float* rgb_ray_out, uint32_t* n_scattered_groups, uint32_t* n_multi_window_groups) {
 	using namespace fused;
+	using GS = StreamGeometry;   // the streaming kernel's sample threads and window
+	using GW = WideGeometry;     // the kernel for the listed groups
 	Args A;
 	A.K = make_loss_const(a);
 	A.n_active = n_rays_counter < a->n_rays ? n_rays_counter : a->n_rays;
 	A.rays_rgba = rays_rgba; A.ray_coord_indices = ray_coord_indices; A.dt_arr = dt; A.coords = coords; A.compacted_coords = compacted_coords;
 	A.net = net; A.dloss = dloss; A.loss_output = loss_output; A.rgb_ray_out = rgb_ray_out; A.mean_density = a->mean_density;
-	const uint32_t n_groups = (a->n_rays + RAYS - 1) / RAYS;
-	uint32_t prefix = *n_compacted_counter;
-	std::vector<SlotState<HI>> st(THREADS);
+	const bool plain = A.K.rgb_act == SRF_ACT_NONE && A.K.density_act == SRF_ACT_NONE;
+	const uint32_t n_groups = (A.n_active + RAYS - 1) / RAYS;
+	std::vector<SlotState<GS, HI>> st_s(GS::THREADS);
+	std::vector<SlotState<GW, HI>> st_w(GW::THREADS);
 	std::vector<RayCarry> c(RAYS);
-	Shared* shp = new Shared();
-	Shared& sh = *shp;
-	Plan& pl = sh.plan;
-	for (uint32_t g = 0; g < n_groups; ++g) {
+	std::vector<uint32_t> side((size_t)n_groups * RAYS, 0);
+	std::vector<uint32_t> slow;
+	Window<GS>* ws = new Window<GS>[2];
+	Window<GW>* ww = new Window<GW>();
+	RayLds* rlp = new RayLds();
+	RayLds& rl = *rlp;
+	Plan plans[NPLAN];
+	auto make_plan = [&](uint32_t g, Plan& pl, std::vector<Float4>* tgt) {
 		const uint32_t ray0 = g * RAYS;
 		pl.misc[M_SUM] = 0; pl.misc[M_CONTIG] = 1;
-		std::vector<Float4> tgt(RAYS);
-		for (uint32_t t = 0; t < RAYS; ++t) load_ray(t, ray0, A, pl, &tgt[t]);
+		Float4 dummy;
+		for (uint32_t t = 0; t < RAYS; ++t) load_ray(t, ray0, A, pl, tgt ? &(*tgt)[t] : &dummy);
 		for (uint32_t t = 0; t < RAYS; ++t) plan_lane(t, ray0, A, pl);
 		for (uint32_t t = 0; t < RAYS; ++t) plan_finish_lane(t, ray0, A, pl);
-		const bool contig = pl.misc[M_CONTIG] != 0;
-		const uint32_t total = pl.misc[M_TOTAL];
-		const uint32_t n_win = (total + WIN - 1) / WIN;
-		if (!contig) ++*n_scattered_groups;
-		if (contig && n_win > 1) ++*n_multi_window_groups;
-		auto sweep = [&](uint32_t win, bool emit) {
-			for (uint32_t t = 0; t < THREADS; ++t) phase_a<HI>(t, win, A, sh, pl, st[t]);
-			for (uint32_t t = 0; t < RAYS; ++t) chain(t, win, A, sh, pl, c[t]);
-			if (emit) for (uint32_t t = 0; t < THREADS; ++t) phase_c<HI, HO>(t, win, A, sh, pl, st[t]);
-		};
-		if (contig) {
-			for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
-			for (uint32_t win = 0; win < n_win; ++win) sweep(win, false);
-			for (uint32_t t = 0; t < RAYS; ++t) finish_ray(t, ray0, A, sh, c[t], tgt[t]);
-		} else {
-			for (uint32_t t = 0; t < RAYS; ++t) {
-				uint32_t n = 0;
-				loss_forward_body<HI>(ray0 + t, A.K, A.rays_rgba, A.n_active, A.ray_coord_indices, A.dt_arr, A.net, &sh.fw[t], &n, A.rgb_ray_out);
-				sh.rnf[t] = n;
-			}
+	};
+	// k_chain_prepare and k_chain_items: the items in ray order, and which of them belong to listed groups
+	std::vector<U2> items;
+	for (uint32_t g = 0; g < n_groups; ++g) {
+		make_plan(g, plans[0], nullptr);
+		const uint32_t word = group_items_word<GS>(plans[0]);
+		U2 it[2];
+		const uint32_t n = items_of_group(g, word, it);
+		if (item_listed(it[0])) {
+			slow.push_back(g);
+			if (plans[0].misc[M_CONTIG] == 0) ++*n_scattered_groups; else ++*n_multi_window_groups;
 		}
-		uint32_t run = prefix;
-		for (uint32_t t = 0; t < RAYS; ++t) {
-			const uint32_t n = sh.rnf[t];
-			if (contig) commit_ray(t, ray0, run, A, sh); else sh.out[t].cbase = run;
-			run += n;
-		}
-		prefix = run;
-		if (contig) {
-			if (n_win == 1) {
-				for (uint32_t t = 0; t < THREADS; ++t) phase_c<HI, HO>(t, 0, A, sh, pl, st[t]);
-			} else if (n_win > 1) {
-				for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
-				for (uint32_t win = 0; win < n_win; ++win) sweep(win, true);
-			}
-		} else {
-			for (uint32_t t = 0; t < RAYS; ++t)
-				loss_backward_body<HI, HO>(ray0 + t, A.K, A.n_active, A.ray_coord_indices, A.dt_arr, A.coords, A.compacted_coords, A.net, A.dloss, A.loss_output,
-				                           A.mean_density, sh.fw[t], sh.rnf[t], sh.out[t].cbase, nullptr);
-		}
+		for (uint32_t k = 0; k < n; ++k) items.push_back(it[k]);
 	}
-	*n_compacted_counter = prefix;
-	delete shp;
-}
-
-
-// The two-pass compositing: forward phases of every group -> exclusive scan of the per-ray counts -> forward phases again
-// plus gradients at the scanned offsets (the device kernel additionally overlaps the next group's loads with the
-// current group's work, which changes no value).
-template <bool HI, bool HO>
-static void run_twopass(const orc_loss_args* a, const float* rays_rgba, uint32_t n_rays_counter, uint32_t* ray_coord_indices, const float* dt,
-                        const float* coords, float* compacted_coords, uint32_t* n_compacted_counter, const void* net, void* dloss, float* loss_output,
-                        float* rgb_ray_out) {
-	using namespace fused;
-	Args A;
-	A.K = make_loss_const(a);
-	A.n_active = n_rays_counter < a->n_rays ? n_rays_counter : a->n_rays;
-	A.rays_rgba = rays_rgba; A.ray_coord_indices = ray_coord_indices; A.dt_arr = dt; A.coords = coords; A.compacted_coords = compacted_coords;
-	A.net = net; A.dloss = dloss; A.loss_output = loss_output; A.rgb_ray_out = nullptr; A.mean_density = a->mean_density;
-	const uint32_t n_groups = (a->n_rays + RAYS - 1) / RAYS;
-	std::vector<uint32_t> n_fwd(a->n_rays, 0), cbase(a->n_rays, 0);
-	std::vector<SlotState<HI>> st(THREADS);
-	std::vector<RayCarry> c(RAYS);
-	Shared* shp = new Shared();
-	Shared& sh = *shp;
-	Plan plan_next;
-	for (int pass = 0; pass < 2; ++pass) {
-		const bool backward = pass == 1;
-		if (backward) {
-			uint32_t run = *n_compacted_counter;
-			for (uint32_t i = 0; i < a->n_rays; ++i) { cbase[i] = run; run += n_fwd[i]; }
-			*n_compacted_counter = run;
-			A.rgb_ray_out = rgb_ray_out;
-		}
-		for (uint32_t g = 0; g < n_groups; ++g) {
-			Plan& pl = (g & 1) ? plan_next : sh.plan;
+	// k_slow_groups, forward and backward
+	auto slow_groups = [&](bool backward) {
+		Args B = A;
+		if (!backward) B.rgb_ray_out = nullptr;
+		Plan& pl = plans[0];
+		for (uint32_t g : slow) {
 			const uint32_t ray0 = g * RAYS;
-			pl.misc[M_SUM] = 0; pl.misc[M_CONTIG] = 1;
 			std::vector<Float4> tgt(RAYS);
-			for (uint32_t t = 0; t < RAYS; ++t) load_ray(t, ray0, A, pl, &tgt[t]);
-			for (uint32_t t = 0; t < RAYS; ++t) plan_lane(t, ray0, A, pl);
-			for (uint32_t t = 0; t < RAYS; ++t) plan_finish_lane(t, ray0, A, pl);
-			const bool contig = pl.misc[M_CONTIG] != 0;
-			const uint32_t total = pl.misc[M_TOTAL];
-			const uint32_t n_win = (total + WIN - 1) / WIN;
-			if (contig) {
+			make_plan(g, pl, &tgt);
+			if (pl.misc[M_CONTIG] != 0) {
+				const uint32_t n_win = (pl.misc[M_TOTAL] + GW::WIN - 1) / GW::WIN;
 				for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
 				for (uint32_t win = 0; win < n_win; ++win) {
-					for (uint32_t t = 0; t < THREADS; ++t) { phase_a_load<HI>(t, win, A, pl, st[t]); }
-					for (uint32_t t = 0; t < THREADS; ++t) { phase_a_compute<HI>(t, win, A, sh, pl, st[t]); }
-					for (uint32_t t = 0; t < RAYS; ++t) chain(t, win, A, sh, pl, c[t]);
+					for (uint32_t t = 0; t < GW::THREADS; ++t) phase_a<GW, HI>(t, win, B, *ww, pl, st_w[t]);
+					for (uint32_t t = 0; t < RAYS; ++t) chain<GW>(t, win, B, *ww, rl, pl, c[t]);
 				}
-				for (uint32_t t = 0; t < RAYS; ++t) finish_ray(t, ray0, A, sh, c[t], tgt[t]);
-				if (backward) {
-					for (uint32_t t = 0; t < RAYS; ++t) commit_ray(t, ray0, ray0 + t < a->n_rays ? cbase[ray0 + t] : 0u, A, sh);
-					if (n_win == 1) {
-						for (uint32_t t = 0; t < THREADS; ++t) phase_c<HI, HO>(t, 0, A, sh, pl, st[t]);
-					} else if (n_win > 1) {
-						for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
-						for (uint32_t win = 0; win < n_win; ++win) {
-							for (uint32_t t = 0; t < THREADS; ++t) phase_a<HI>(t, win, A, sh, pl, st[t]);
-							for (uint32_t t = 0; t < RAYS; ++t) chain(t, win, A, sh, pl, c[t]);
-							for (uint32_t t = 0; t < THREADS; ++t) phase_c<HI, HO>(t, win, A, sh, pl, st[t]);
-						}
-					}
+				for (uint32_t t = 0; t < RAYS; ++t) finish_ray(t, ray0, B, rl, c[t], tgt[t]);
+				if (!backward) {
+					for (uint32_t t = 0; t < RAYS; ++t) if (ray0 + t < B.n_active) side[ray0 + t] = rl.rnf[t];
 				} else {
-					for (uint32_t t = 0; t < RAYS; ++t) if (ray0 + t < a->n_rays) n_fwd[ray0 + t] = sh.rnf[t];
+					for (uint32_t t = 0; t < RAYS; ++t) commit_ray(t, ray0, ray0 + t < B.n_active ? side[ray0 + t] : 0u, B, rl);
+					for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
+					for (uint32_t win = 0; win < n_win; ++win) {
+						for (uint32_t t = 0; t < GW::THREADS; ++t) phase_a<GW, HI>(t, win, B, *ww, pl, st_w[t]);
+						for (uint32_t t = 0; t < RAYS; ++t) chain<GW>(t, win, B, *ww, rl, pl, c[t]);
+						for (uint32_t t = 0; t < GW::THREADS; ++t) phase_c<GW, HI, HO>(t, win, B, *ww, rl, pl, st_w[t]);
+					}
 				}
 			} else {
 				for (uint32_t t = 0; t < RAYS; ++t) {
 					uint32_t n = 0;
-					loss_forward_body<HI>(ray0 + t, A.K, A.rays_rgba, A.n_active, A.ray_coord_indices, A.dt_arr, A.net, &sh.fw[t], &n, A.rgb_ray_out);
-					if (backward) loss_backward_body<HI, HO>(ray0 + t, A.K, A.n_active, A.ray_coord_indices, A.dt_arr, A.coords, A.compacted_coords, A.net, A.dloss,
-					                                         A.loss_output, A.mean_density, sh.fw[t], n, ray0 + t < a->n_rays ? cbase[ray0 + t] : 0u, nullptr);
-					else if (ray0 + t < a->n_rays) n_fwd[ray0 + t] = n;
+					FwdRay fw;
+					loss_forward_body<HI>(ray0 + t, B.K, B.rays_rgba, B.n_active, B.ray_coord_indices, B.dt_arr, B.net, &fw, &n, B.rgb_ray_out);
+					if (ray0 + t >= B.n_active) continue;
+					if (!backward) side[ray0 + t] = n;
+					else loss_backward_body<HI, HO>(ray0 + t, B.K, B.n_active, B.ray_coord_indices, B.dt_arr, B.coords, B.compacted_coords, B.net, B.dloss, B.loss_output,
+					                                B.mean_density, fw, n, side[ray0 + t], nullptr);
 				}
 			}
 		}
+	};
+	slow_groups(false);
+	// k_composite_stream (items in order and one at a time; the device spreads them over persistent workgroups and
+	// keeps three of a workgroup's items under way in two windows)
+	uint32_t prefix = *n_compacted_counter;
+	Plan group_plan;
+	for (size_t i = 0; i < items.size(); ++i) {
+		const U2 item = items[i];
+		const uint32_t g = item.x, ray0 = g * RAYS, lo = item_lo(item), hi = item_hi(item);
+		std::vector<Float4> tgt(RAYS);
+		make_plan(g, group_plan, &tgt);
+		Plan& pl = plans[i % NPLAN];
+		Window<GS>& w = ws[i % 2];
+		for (uint32_t t = 0; t < RAYS; ++t) plan_part_lane(t, group_plan, lo, hi, g, pl);
+		const bool fast = !item_listed(item);
+		std::vector<uint32_t> n(RAYS, 0);
+		if (fast) {
+			for (uint32_t t = 0; t < GS::THREADS; ++t) phase_a_load_single<GS, HI>(t, A, pl, st_s[t]);
+			for (uint32_t t = 0; t < GS::THREADS; ++t) { if (plain) phase_a_compute<GS, HI, true>(t, 0, A, w, pl, st_s[t]); else phase_a_compute<GS, HI, false>(t, 0, A, w, pl, st_s[t]); }
+			uint32_t rn_max = 0, n_max = 0;
+			for (uint32_t t = 0; t < RAYS; ++t) rn_max = pl.rn[t] > rn_max ? pl.rn[t] : rn_max;
+			for (uint32_t t = 0; t < RAYS; ++t) n[t] = count_lane<GS>(t, rn_max, A, w, pl);
+			for (uint32_t t = 0; t < RAYS; ++t) n_max = n[t] > n_max ? n[t] : n_max;
+			for (uint32_t t = 0; t < RAYS; ++t) chain_counted<GS>(t, n[t], n_max, w, rl, pl, c[t]);
+			for (uint32_t t = 0; t < RAYS; ++t) finish_ray(t, ray0, A, rl, c[t], tgt[t], lo, hi);
+		} else {
+			for (uint32_t t = 0; t < RAYS; ++t) n[t] = ray0 + t < A.n_active ? side[ray0 + t] : 0u;
+		}
+		uint32_t run = prefix;
+		for (uint32_t t = 0; t < RAYS; ++t) {
+			if (fast) commit_ray(t, ray0, run, A, rl, lo, hi);
+			else if (ray0 + t < A.n_active) side[ray0 + t] = run;
+			run += n[t];
+		}
+		prefix = run;
+		if (fast) {
+			for (uint32_t t = 0; t < GS::THREADS; ++t) { if (plain) phase_c<GS, HI, HO, true, false>(t, 0, A, w, rl, pl, st_s[t]); else phase_c<GS, HI, HO, false, false>(t, 0, A, w, rl, pl, st_s[t]); }
+			if (A.compacted_coords) for (uint32_t q0 = 0; q0 < pl.misc[M_TOTAL]; q0 += COORDS_DEPTH * RAYS) for (uint32_t t = 0; t < RAYS; ++t) coords_copy_rows<GS>(t, q0, A, w, rl, pl);
+		}
 	}
-	delete shp;
+	*n_compacted_counter = prefix;
+	slow_groups(true);
+	delete[] ws; delete ww; delete rlp;
 }
 
 extern "C" {
@@ -547,14 +537,6 @@ void hs_loss_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n_ra
 #undef RUN
 }
 
-void hs_loss_twopass(const orc_loss_args* a, const float* rays_rgba, uint32_t n_rays_counter, uint32_t* ray_coord_indices, const float* dt,
-                     const float* coords, float* compacted_coords, uint32_t* n_compacted_counter, const void* net, void* dloss, float* loss_output,
-                     float* rgb_ray_out) {
-	const bool hin = a->network_output_dtype == ORC_DTYPE_F16, hout = a->dloss_dtype == ORC_DTYPE_F16;
-#define RUN(HI, HO) run_twopass<HI, HO>(a, rays_rgba, n_rays_counter, ray_coord_indices, dt, coords, compacted_coords, n_compacted_counter, net, dloss, loss_output, rgb_ray_out)
-	if (hin && hout) RUN(true, true); else if (hin) RUN(true, false); else if (hout) RUN(false, true); else RUN(false, false);
-#undef RUN
-}
 
 void hs_volume_rendering(const orc_params* p, const orc_render_args* a, srf_ray_payload* payloads, float* rgba, const float* coords, const void* net) {
 	const Params P = to_params(p);

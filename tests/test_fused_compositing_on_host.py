@@ -19,6 +19,9 @@ def layout(rng, kind, n_rays):
         counts = rng.integers(0, 60, n_rays)
         counts[rng.random(n_rays) < 0.03] = rng.integers(2000, 5000)
         counts[5] = 4097
+    elif kind == "split":        # groups longer than one window of the streaming kernel, cut at a ray boundary into two parts
+        counts = rng.integers(25, 60, n_rays)
+        counts[n_rays // 3:n_rays // 3 + 40] = rng.integers(0, 12, 40)
     elif kind == "tiny":
         counts = rng.integers(0, 3, n_rays)
     else:
@@ -37,10 +40,10 @@ def layout(rng, kind, n_rays):
     return counts.astype(np.uint32), base.astype(np.uint32), total
 
 
-@pytest.mark.parametrize("kind", ["short", "long", "tiny", "gaps", "biggap", "shuffled"])
+@pytest.mark.parametrize("kind", ["short", "long", "split", "tiny", "gaps", "biggap", "shuffled"])
 @pytest.mark.parametrize("hin,hout", [(False, False), (True, False), (True, True)])
 def test_fused_equals_oracle(orc, hostsim, kind, hin, hout):
-    rng = np.random.default_rng(["short", "long", "tiny", "gaps", "biggap", "shuffled"].index(kind) + 100)
+    rng = np.random.default_rng(["short", "long", "tiny", "gaps", "biggap", "shuffled", "split"].index(kind) + 100)
     n_rays = 64 * 5 + 17
     counts, base, total = layout(rng, kind, n_rays)
     net = helpers.random_network_output(rng, total, np.float16 if hin else np.float32)
@@ -54,7 +57,7 @@ def test_fused_equals_oracle(orc, hostsim, kind, hin, hout):
               background_color=(O.f32 * 3)(0.1, 0.7, 0.3), mean_density=0.001)
     a = loss_args(n_rays, cap, **kw)
     outs = []
-    for fn in ("oracle", "fused", "twopass"):
+    for fn in ("oracle", "fused"):
         idx = np.stack([counts, base], axis=1).astype(np.uint32)
         dloss = np.zeros((cap, 4), np.float16 if hout else np.float32)
         comp = np.zeros((cap, 7), np.float32)
@@ -65,11 +68,6 @@ def test_fused_equals_oracle(orc, hostsim, kind, hin, hout):
         if fn == "oracle":
             tot = orc.volume_rendering_with_loss_and_gradient(a, tgt, n_active, idx, dt, net, dloss, n_compacted_counter=11, coords=coords,
                                                               compacted_coords=comp, loss_output=loss, rgb_ray_out=rgb)
-        elif fn == "twopass":
-            cnt = np.array([11], np.uint32)
-            hostsim.lib.hs_loss_twopass(C.byref(a), ptr(tgt), n_active, ptr(idx), ptr(dt), ptr(coords), ptr(comp), ptr(cnt), ptr(net), ptr(dloss),
-                                        ptr(loss), ptr(rgb))
-            tot = int(cnt[0])
         else:
             cnt = np.array([11], np.uint32)
             ns, nm = C.c_uint32(), C.c_uint32()
@@ -97,17 +95,13 @@ def test_fused_handles_empty_and_inactive_batches(orc, hostsim):
         tgt = rng.random((n_rays, 4)).astype(np.float32)
         a = loss_args(n_rays, max(total, 1))
         res = []
-        for fn in ("oracle", "fused", "twopass"):
+        for fn in ("oracle", "fused"):
             idx = np.stack([counts, base], axis=1).astype(np.uint32)
             dloss = np.zeros((max(total, 1), 4), np.float32)
             loss = np.full(n_rays, -1, np.float32)
             rgb = np.zeros((n_rays, 3), np.float32)
             if fn == "oracle":
                 tot = orc.volume_rendering_with_loss_and_gradient(a, tgt, n_active, idx, dt, net, dloss, loss_output=loss, rgb_ray_out=rgb)
-            elif fn == "twopass":
-                cnt = np.array([0], np.uint32)
-                hostsim.lib.hs_loss_twopass(C.byref(a), ptr(tgt), n_active, ptr(idx), ptr(dt), None, None, ptr(cnt), ptr(net), ptr(dloss), ptr(loss), ptr(rgb))
-                tot = int(cnt[0])
             else:
                 cnt = np.array([0], np.uint32)
                 ns, nm = C.c_uint32(), C.c_uint32()

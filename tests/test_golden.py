@@ -90,7 +90,7 @@ def test_gpu_reproduces_march_fixture(gpu, name):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("impl", ["twopass", "lookback", "unfused"])
+@pytest.mark.parametrize("impl", ["stream", "unfused"])
 def test_gpu_reproduces_composite_fixture(gpu, impl, monkeypatch):
     torch = gpu
     from sphericalrf_amd import api

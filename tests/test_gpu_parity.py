@@ -369,7 +369,7 @@ def test_render_loop_and_fused_frame(gpu, orc, config_id, scale):
         prev, cur = dbi % 2, (dbi + 1) % 2
         dbi += 1
         n_alive_t.zero_()
-        api.compact_rays(n_alive, pay[prev], col[prev], pay[cur], col[cur], hit_p, hit_c, n_alive_t, n_hit)
+        api.compact_rays(m, n_alive, pay[prev], col[prev], pay[cur], col[cur], hit_p, hit_c, n_alive_t, n_hit)
         n_alive = int(n_alive_t.item())
         if n_alive == 0:
             break
@@ -465,24 +465,29 @@ def test_errors_are_reported_not_thrown_across_the_abi(gpu):
         s.init(1, (4, 4), (1.0, 1.0), (0.5, 0.5), None, None, api.Pcg32(1))
 
 
-@pytest.mark.parametrize("impl", ["twopass", "lookback"])
-@pytest.mark.parametrize("kind", ["short", "long", "tiny", "gaps", "biggap", "shuffled"])
-def test_single_launch_compositing_layouts(gpu, orc, kind, impl, monkeypatch):
-    """every sample layout the group-wise kernels distinguish, against the oracle, for the two-pass implementation and for
-    the single-launch one (many workgroups, so its ordered offsets really go through the look-back chain)"""
-    monkeypatch.setenv("SRF_COMPOSITE_IMPL", impl)
+@pytest.mark.parametrize("acts", ["plain", "activated"])
+@pytest.mark.parametrize("kind", ["short", "long", "split", "tiny", "gaps", "biggap", "shuffled"])
+def test_single_launch_compositing_layouts(gpu, orc, kind, acts, monkeypatch):
+    """every sample layout the streaming compositing distinguishes (back-to-back rays, holes, groups longer than a window,
+    shuffled offsets), against the oracle, over many workgroups so that its ordered offsets really go through the chain;
+    with the activations compiled out ("plain": both None) and with the run-time switches (Logistic colour, Exponential density)"""
+    monkeypatch.delenv("SRF_COMPOSITE_IMPL", raising=False)
+    rgb_act, den_act = (O.ACT_NONE, O.ACT_NONE) if acts == "plain" else (O.ACT_LOGISTIC, O.ACT_EXPONENTIAL)
     torch = gpu
     from sphericalrf_amd import api
     from tests.test_fused_compositing_on_host import layout
-    rng = np.random.default_rng(["short", "long", "tiny", "gaps", "biggap", "shuffled"].index(kind) + 200)
+    rng = np.random.default_rng(["short", "long", "tiny", "gaps", "biggap", "shuffled", "split"].index(kind) + 200)
     n_rays = 64 * 700 + 29
     counts, base, total = layout(rng, kind, n_rays)
     net = helpers.random_network_output(rng, total, np.float16)
     net[:, 3] *= np.float16(0.05 if kind == "long" else 3)
+    if acts == "activated":
+        net[:, 3] = np.log(net[:, 3].astype(np.float32) + 1e-3).astype(np.float16)      # the exponential brings the densities back
     dt = (rng.random(total) * 0.3 + 0.01).astype(np.float32)
     tgt = rng.random((n_rays, 4)).astype(np.float32)
     cap = int(counts.sum() * 0.9) + 1
-    a = loss_args(n_rays, cap, network_output_dtype=O.DTYPE_F16, background_color=(O.f32 * 3)(0.1, 0.7, 0.3), mean_density=0.001)
+    a = loss_args(n_rays, cap, network_output_dtype=O.DTYPE_F16, background_color=(O.f32 * 3)(0.1, 0.7, 0.3), mean_density=0.001,
+                  rgb_activation=rgb_act, density_activation=den_act)
     idx = np.stack([counts, base], axis=1).astype(np.uint32)
     o_idx, o_dloss = idx.copy(), np.zeros((cap, 4), np.float32)
     o_loss, o_rgb = np.full(n_rays, -1, np.float32), np.zeros((n_rays, 3), np.float32)
@@ -498,7 +503,7 @@ def test_single_launch_compositing_layouts(gpu, orc, kind, impl, monkeypatch):
         d_idx.copy_(torch.from_numpy(idx.view(np.int32)))
         cnt.fill_(11)
         m.volume_rendering_with_loss_and_gradient(n_rays, cap, torch.from_numpy(tgt).cuda(), nrc, d_idx, torch.from_numpy(dt).cuda(), torch.from_numpy(net).cuda(), d_dloss, cnt,
-                                                  rgb_activation=api.ACT_NONE, density_activation=api.ACT_NONE, loss_output=d_loss, loss_type="L2", loss_scale=128.0,
+                                                  rgb_activation=rgb_act, density_activation=den_act, loss_output=d_loss, loss_type="L2", loss_scale=128.0,
                                                   density_grid_mean=mean_t, use_grid=True, background_color=(0.1, 0.7, 0.3), rgb_ray_out=d_rgb)
         m.sync_check()
         assert int(cnt.item()) == o_total
@@ -508,9 +513,9 @@ def test_single_launch_compositing_layouts(gpu, orc, kind, impl, monkeypatch):
 
 
 def test_single_launch_and_three_launch_compositing_agree_at_full_size(gpu, orc, monkeypatch):
-    """2^20 rays / ~1.5e7 samples: the two-pass, the single-launch and the one-thread-per-ray implementations (the
-    distortion regulariser forces the last) must give identical results, side buffer of the regulariser aside, and
-    those results are the oracle's"""
+    """2^20 rays / ~1.5e7 samples: the streaming implementation and the one-thread-per-ray implementation (selected by the
+    environment at creation, or forced by the distortion regulariser) must give identical results, side buffer of the
+    regulariser aside, and those results are the oracle's"""
     torch = gpu
     from sphericalrf_amd import api
     g = torch.Generator(device="cuda")
@@ -528,7 +533,7 @@ def test_single_launch_and_three_launch_compositing_agree_at_full_size(gpu, orc,
     nrc = torch.full((1,), n_rays, dtype=torch.int32, device="cuda")
     mean_t = torch.ones(1, device="cuda")
     outs = []
-    for reg, impl in (("None", "twopass"), ("None", "lookback"), ("Distortion", "twopass")):
+    for reg, impl in (("None", "unfused"), ("None", "stream"), ("Distortion", "stream")):
         monkeypatch.setenv("SRF_COMPOSITE_IMPL", impl)
         m = api.RayMarcher(dict(train_with_random_bg_color=False, train_in_linear_color=True, regularization_type=reg))
         idx = idx0.clone()

@@ -5,6 +5,7 @@ import numpy as np
 import pytest
 
 from oracle import oracle as O
+from sphericalrf_amd import scene
 from tests import helpers
 
 
@@ -258,3 +259,137 @@ def test_compact_and_shade(orc):
     for k, src in enumerate([1, 5, 7, 11]):
         px = int(pay["idx"][src])
         assert np.allclose(frame[px], rgba[src] + 0.5 * (1 - rgba[src, 3]))
+
+
+def _unwarp_sinusoidal64(w):
+    """common_device.h:508-520 in float64: inverse of the effective ("ERP" falls through to sinusoidal) warp"""
+    phi = (w[1] - 0.5) * math.pi
+    theta = (w[0] - 0.5) * 2 * math.pi / math.cos(phi)
+    rho = 2 * w[2]
+    rho = rho if rho <= 1 else 1 / (2 - rho)
+    return np.array([rho * math.cos(phi) * math.cos(theta) + 0.5, rho * math.cos(phi) * math.sin(theta) + 0.5, rho * math.sin(phi) + 0.5])
+
+
+@pytest.mark.parametrize("mode", [O.RENDER_AO, O.RENDER_DEPTH, O.RENDER_DISTANCE, O.RENDER_NORMALS, O.RENDER_SHADE])
+def test_inference_render_modes_against_float64_formulas(orc, mode):
+    """ray_marcher.cu:233-281 per render mode: what replaces the colour (alpha for AO, forward distance for Depth, Euclidean
+    distance for Distance, the unit vector along -sigma' * warped_pos for Normals), early stop at alpha sum > 1 - thr, the ray
+    killed with n_steps = j + offset when it consumed fewer than n_steps samples, and the un-normalised accumulator stored"""
+    rng = np.random.default_rng(21 + mode)
+    p = orc.params(aabb_scale=8, warping_type=O.WARP_ERP)
+    n_rays, n_steps = 7, 6
+    net = helpers.random_network_output(rng, n_rays * n_steps).reshape(n_rays, n_steps, 4)
+    net[2, :, 3] *= 40          # ray 2 saturates early
+    coords = np.zeros((n_rays, n_steps, 7), np.float32)
+    coords[..., 0:3] = (rng.random((n_rays, n_steps, 3)) * 0.6 + 0.2).astype(np.float32)
+    coords[..., 3] = (rng.random((n_rays, n_steps)) * 0.3 + 0.05).astype(np.float32)
+    pay = np.zeros(n_rays, O.PAYLOAD_DTYPE)
+    pay["alive"] = 1
+    pay["alive"][5] = 0                                   # a dead ray is left alone
+    pay["n_steps"] = [6, 6, 6, 4, 6, 6, 0]                # ray 3 got only 4 samples, ray 6 none
+    pay["o"] = (rng.random((n_rays, 3)) * 0.2 + 0.4).astype(np.float32)
+    rgba = (rng.random((n_rays, 4)) * 0.1).astype(np.float32)     # accumulators carried in from earlier chunks
+    rgba0 = rgba.copy()
+    cam = scene.look_at(np.array([0.4, 0.5, 0.6]), np.array([0.3, -0.5, 0.2]))
+    a = O.RenderArgs()
+    a.n_rays, a.n_steps, a.n_steps_offset, a.padded_output_width = n_rays, n_steps, 9, 4
+    a.density_activation, a.rgb_activation, a.render_mode = O.ACT_EXPONENTIAL, O.ACT_LOGISTIC, mode
+    a.camera = (O.f32 * 12)(*cam)
+    a.depth_scale, a.transmittance_threshold, a.network_output_dtype = 0.7, 1e-2, O.DTYPE_F32
+    net[..., 3] = np.log(net[..., 3])                     # exponential activation brings the densities back
+    orc.volume_rendering(p, a, pay, rgba, coords, np.ascontiguousarray(net))
+    fwd = cam[6:9].astype(np.float64)
+    for r in range(n_rays):
+        if r == 5:
+            assert np.array_equal(rgba[r], rgba0[r]) and pay["n_steps"][r] == 6 and not pay["alive"][r]
+            continue
+        acc = rgba0[r].astype(np.float64)
+        n_in = [6, 6, 6, 4, 6, 6, 0][r]
+        j = 0
+        while j < n_in:
+            sigma = math.exp(float(net[r, j, 3]))
+            dt = float(coords[r, j, 3])
+            alpha = 1 - math.exp(-sigma * dt)
+            w = alpha * (1 - acc[3])
+            wp = coords[r, j, :3].astype(np.float64)
+            if mode == O.RENDER_SHADE:
+                c = 1 / (1 + np.exp(-net[r, j, :3].astype(np.float64)))
+            elif mode == O.RENDER_AO:
+                c = np.full(3, alpha)
+            elif mode == O.RENDER_NORMALS:
+                v = -math.exp(min(15.0, max(-15.0, float(net[r, j, 3])))) * wp
+                c = v / np.linalg.norm(v)
+            else:
+                rel = _unwarp_sinusoidal64(wp) - pay["o"][r].astype(np.float64)
+                z = (fwd @ rel if mode == O.RENDER_DEPTH else np.linalg.norm(rel)) * 0.7
+                c = np.full(3, z)
+            acc[:3] += c * w
+            acc[3] += w
+            if acc[3] > 1 - 1e-2:
+                break
+            j += 1
+        assert np.allclose(rgba[r], acc, rtol=2e-5, atol=1e-6), (mode, r)
+        if j < n_steps:
+            assert not pay["alive"][r] and pay["n_steps"][r] == j + 9
+        else:
+            assert pay["alive"][r] and pay["n_steps"][r] == 6
+    assert not pay["alive"][2] and pay["n_steps"][2] < 6 + 9         # the saturated ray stopped early
+    assert not pay["alive"][3] and pay["n_steps"][3] == 4 + 9        # ran out of samples
+    assert not pay["alive"][6] and pay["n_steps"][6] == 0 + 9
+
+
+def test_shade_modes_against_float64_formulas(orc):
+    """testbed.cu:448-477: Normals maps the normalised accumulated vector to 0.5 n + 0.5 times alpha, Cost shows n_steps / 128
+    with alpha 1, Shade converts sRGB to linear unless training is in linear colours; then tmp + frame * (1 - tmp.w)"""
+    rng = np.random.default_rng(33)
+    n = 9
+    pay = np.zeros(n, O.PAYLOAD_DTYPE)
+    pay["idx"] = rng.permutation(n)
+    pay["n_steps"] = rng.integers(0, 400, n)
+    rgba = rng.random((n, 4)).astype(np.float32)
+    rgba[0, :3] = [0.001, 0.03, 0.5]            # both branches of srgb_to_linear
+    frame0 = rng.random((n, 4)).astype(np.float32)
+
+    def srgb_to_linear(v):
+        return v / 12.92 if v <= 0.04045 else ((v + 0.055) / 1.055) ** 2.4
+
+    for mode, linear in ((O.RENDER_NORMALS, True), (O.RENDER_COST, False), (O.RENDER_SHADE, False), (O.RENDER_SHADE, True), (O.RENDER_DEPTH, False)):
+        frame = frame0.copy()
+        orc.shade(n, rgba, pay, frame, mode, linear)
+        for i in range(n):
+            tmp = rgba[i].astype(np.float64)
+            if mode == O.RENDER_NORMALS:
+                v = tmp[:3] / np.linalg.norm(tmp[:3])
+                tmp[:3] = (0.5 * v + 0.5) * tmp[3]
+            elif mode == O.RENDER_COST:
+                tmp = np.array([pay["n_steps"][i] / 128.0] * 3 + [1.0])
+            if not linear and mode == O.RENDER_SHADE:
+                tmp[:3] = [srgb_to_linear(v) for v in tmp[:3]]
+            want = tmp + frame0[pay["idx"][i]].astype(np.float64) * (1 - tmp[3])
+            assert np.allclose(frame[pay["idx"][i]], want, rtol=1e-5, atol=1e-7), (mode, linear, i)
+
+
+def test_distortion_side_buffer_holds_running_sums_with_unit_transmittance(orc):
+    """ray_marcher.cu:142-166: per compacted sample the running sum of alpha (T stays 1 in that loop) and of alpha (j+1)/n"""
+    rng = np.random.default_rng(17)
+    counts = [5, 3, 6]
+    n = sum(counts)
+    net = helpers.random_network_output(rng, n)
+    dt = (rng.random(n) * 0.3 + 0.05).astype(np.float32)
+    tgt = rng.random((3, 4)).astype(np.float32)
+    a = loss_args(3, 100, transmittance_threshold=0.0, regularization_type=O.REG_DISTORTION)
+    idx = np.zeros((3, 2), np.uint32)
+    idx[:, 0] = counts
+    idx[:, 1] = np.concatenate([[0], np.cumsum(counts)[:-1]])
+    reg = np.zeros((100, 2), np.float32)
+    dloss = np.zeros((100, 4), np.float32)
+    orc.volume_rendering_with_loss_and_gradient(a, tgt, 3, idx, dt, net, dloss, reg_buffer=reg)
+    k = 0
+    for c in counts:
+        sw = swp = 0.0
+        for j in range(c):
+            alpha = 1 - math.exp(-float(net[k, 3]) * float(dt[k]))
+            sw += alpha
+            swp += alpha * (j + 1) / c
+            assert abs(reg[k, 0] - sw) < 1e-5 and abs(reg[k, 1] - swp) < 1e-5
+            k += 1

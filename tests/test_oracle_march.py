@@ -208,3 +208,114 @@ def test_render_rays_match_one_uninterrupted_march(orc):
     a, b, c = ([until_stuck(r) for r in s] for s in seqs)
     assert a == b == c
     assert sum(len(r) for r in a) > 0
+
+
+def _hand_walk_until_occupied(orc, p, bf, o, d, t):
+    """occupancy_sampler.cu:773-794 / :827-853 by hand with the oracle's scalar helpers: returns (t, state, dt) where state
+    is "occupied" (stopped at an occupied step, t not advanced), "outside" (left the box) or "stuck" (dt == 0 after t += dt)"""
+    for _ in range(100000):
+        pos = (o + t * d).astype(np.float32)
+        if not orc.contains(p, pos):
+            return t, "outside", np.float32(0)
+        dt = orc.calc_dt(p, t)
+        w = orc.warp_position(p, pos)
+        lvl = orc.level_from_pos(p, pos, w)
+        if orc.occupied_at(p, bf, pos, w, lvl):
+            return t, "occupied", dt
+        t = np.float32(t + dt)
+        if dt == 0:
+            return t, "stuck", dt
+    raise AssertionError("walk did not end")
+
+
+def test_render_rays_walked_by_hand(orc):
+    """advance_pos and generate_coords_from_rays against a step-by-step walk written from occupancy_sampler.cu:691-863:
+    start t = max(tmin, 0.05) + 1e-6, jitter ld_random_val(spp, i * 786433) * calc_dt(t0), stop AT the first occupied
+    step, alive flag cleared when the ray leaves the box or the step collapses at the far plane, then n_steps samples
+    per call, each {warp(pos), dt, (d + 1) / 2}, with t stored only when all n_steps were emitted."""
+    res = (6, 5)
+    p, ds, cams, _, _ = small_setup(orc, N=8, C=2, n_max_steps=48, res=res)
+    f = scene.focal_from_fov(res[0], 60.0)
+    rng = np.random.default_rng(11)
+    bf = rng.integers(0, 256, p.n_total // 8).astype(np.uint8) & rng.integers(0, 256, p.n_total // 8).astype(np.uint8) & rng.integers(0, 256, p.n_total // 8).astype(np.uint8)
+    for spp in (0, 3):
+        pay = orc.init_rays_with_payload(p, res, (f, f), (0.5, 0.5), cams[1], spp=spp)
+        n = pay.size
+        assert n == 30 and pay["alive"].all()
+        o_all, d_all, t0_all = pay["o"].copy(), pay["d"].copy(), pay["t"].copy()
+        for i in range(n):
+            tmin = orc.ray_intersect(p, o_all[i], d_all[i])[0]
+            assert t0_all[i] == np.float32(np.float32(max(tmin, np.float32(0.05))) + np.float32(1e-6))
+            assert pay["idx"][i] == i and pay["n_steps"][i] == 0
+        orc.advance_pos(p, pay, bf, spp=spp)
+        walked = []
+        for i in range(n):
+            t0 = t0_all[i]
+            start = np.float32(t0 + np.float32(np.float32(orc.ld_random_val(spp, (i * 786433) & 0xffffffff)) * orc.calc_dt(p, t0)))
+            t, state, dt = _hand_walk_until_occupied(orc, p, bf, o_all[i], d_all[i], start)
+            walked.append((t, state))
+            assert pay["t"][i] == t, (i, pay["t"][i], t)
+            assert bool(pay["alive"][i]) == (state == "occupied")
+        assert any(s == "occupied" for _, s in walked) and any(s != "occupied" for _, s in walked)
+        # the jitter really is there: some start differs from t0
+        assert any(np.float32(orc.ld_random_val(spp, (i * 786433) & 0xffffffff)) != 0 for i in range(n))
+
+        n_steps = 3
+        coords = np.full((n, n_steps, 7), np.nan, np.float32)
+        before = pay.copy()
+        orc.generate_coords_from_rays(p, n, n_steps, bf, pay, coords)
+        n_checked = 0
+        for i in range(n):
+            if not before["alive"][i]:
+                assert pay["t"][i] == before["t"][i] and np.isnan(coords[i]).all()
+                continue
+            t = before["t"][i]
+            emitted, ended = [], False
+            for j in range(n_steps):
+                t, state, dt = _hand_walk_until_occupied(orc, p, bf, o_all[i], d_all[i], t)
+                if state != "occupied":
+                    ended = True
+                    break
+                pos = (o_all[i] + t * d_all[i]).astype(np.float32)
+                emitted.append(np.concatenate([orc.warp_position(p, pos), [dt], ((d_all[i] + np.float32(1)) * np.float32(0.5)).astype(np.float32)]).astype(np.float32))
+                t = np.float32(t + dt)
+            k = len(emitted)
+            assert pay["n_steps"][i] == k
+            assert np.array_equal(coords[i, :k], np.array(emitted, np.float32).reshape(k, 7))
+            assert np.isnan(coords[i, k:]).all()              # nothing is written past the last sample
+            if ended:
+                assert pay["t"][i] == before["t"][i]          # the kernel returns without storing t
+                assert k < n_steps
+            else:
+                assert pay["t"][i] == t
+            assert pay["alive"][i]                            # this kernel never clears the flag (volume_rendering does)
+            n_checked += k
+        assert n_checked > 10
+
+
+def test_render_ray_that_starts_outside_the_box_is_dead(orc):
+    """a camera outside the box looking away: ray_intersect gives {1e5, 1e5}-like misses and o + t d is not contained"""
+    res = (4, 4)
+    p, ds, cams, _, _ = small_setup(orc, N=8, C=1, res=res)
+    f = scene.focal_from_fov(res[0], 60.0)
+    cam = scene.look_at(np.array([0.5 + 100.0, 0.5, 0.5]), np.array([1.0, 0.0, 0.0]))
+    pay = orc.init_rays_with_payload(p, res, (f, f), (0.5, 0.5), cam)
+    assert not pay["alive"].any()
+    assert np.array_equal(pay["o"], np.tile(cam[9:12], (16, 1)))
+    bf = np.full(p.n_total // 8, 0xff, np.uint8)
+    before = pay.copy()
+    orc.advance_pos(p, pay, bf)
+    assert np.array_equal(pay.view(np.uint8), before.view(np.uint8))
+
+
+def test_render_ray_reaching_far_inside_empty_space_dies_with_dt_zero(orc):
+    """far plane inside the box, nothing occupied: the disparity step collapses to 0 at t >= far and advance_pos clears the flag"""
+    res = (3, 3)
+    p, ds, cams, _, _ = small_setup(orc, N=8, C=1, res=res, n_max_steps=16)
+    f = scene.focal_from_fov(res[0], 60.0)
+    bf = np.zeros(p.n_total // 8, np.uint8)
+    pay = orc.init_rays_with_payload(p, res, (f, f), (0.5, 0.5), cams[0])
+    orc.advance_pos(p, pay, bf)
+    assert not pay["alive"].any()
+    assert (pay["t"] >= np.float32(p.far_distance)).all() and (pay["t"] < np.float32(p.far_distance) + 1).all()
+    assert all(orc.calc_dt(p, t) == 0 for t in pay["t"])
