@@ -222,6 +222,22 @@ int  srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const
         const void* network_output, void* dloss_doutput, float* loss_output,
         const float* density_grid_mean, float* rgb_ray_out, void* stream);
 
+/*
+ * The same call for callers that must not allocate device memory while they run (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It runs the single-launch implementation with its
+ * scratch (the per-item status words, item lists and per-ray side array of the ordered-offset chain) in an array that is part of
+ * the library's device image, about 1.3 MB on every GPU the library runs on, and calls no hipMalloc / hipFree.
+ * Limits: n_rays <= SRF_NOALLOC_MAX_RAYS; no distortion regulariser; refused on a marcher that has fallen back to the
+ * three-launch implementation.  All calls on one GPU share the array: calls that overlap on one GPU (different streams or
+ * threads) race.  Arguments, results and error reporting are those of srf_marcher_volume_rendering_with_loss_and_gradient.
+ */
+#define SRF_NOALLOC_MAX_RAYS 262144u
+int  srf_marcher_volume_rendering_with_loss_and_gradient_noalloc(srf_marcher_t* m, const srf_loss_args* args,
+        const float* rays_rgba, const uint32_t* n_rays_counter, uint32_t* ray_coord_indices,
+        const float* dt, const float* coords, float* compacted_coords, uint32_t* n_compacted_coords_counter,
+        const void* network_output, void* dloss_doutput, float* loss_output,
+        const float* density_grid_mean, float* rgb_ray_out, void* stream);
+
 typedef struct srf_render_args {
 	uint32_t n_rays, n_steps, i_steps_offset;
 	uint32_t padded_output_width;

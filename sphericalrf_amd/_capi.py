@@ -93,7 +93,7 @@ SYMBOLS = [
     "srf_sampler_update_grid_bitfield", "srf_sampler_sample_coords_from_dataset", "srf_sampler_generate_rays_from_camera_matrix",
     "srf_sampler_generate_coords_from_rays",
     "srf_marcher_config_default", "srf_marcher_create", "srf_marcher_destroy", "srf_marcher_get_config", "srf_marcher_set_config",
-    "srf_marcher_volume_rendering_with_loss_and_gradient", "srf_marcher_sync_check", "srf_marcher_volume_rendering",
+    "srf_marcher_volume_rendering_with_loss_and_gradient", "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc", "srf_marcher_sync_check", "srf_marcher_volume_rendering",
     "srf_compact_rays", "srf_shade", "srf_fill_rollover", "srf_fill_rollover_and_rescale",
     "srf_render_frame_fused", "srf_field_eval", "srf_debug_eval_elem", "srf_marcher_debug_set_lookback_spin_limit",
 ]
@@ -145,6 +145,7 @@ def load():
     L.srf_marcher_get_config.argtypes = [vp, P(MarcherConfig)]
     L.srf_marcher_set_config.argtypes = [vp, P(MarcherConfig)]
     L.srf_marcher_volume_rendering_with_loss_and_gradient.argtypes = [vp, P(LossArgs), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    L.srf_marcher_volume_rendering_with_loss_and_gradient_noalloc.argtypes = L.srf_marcher_volume_rendering_with_loss_and_gradient.argtypes
     L.srf_marcher_sync_check.argtypes = [vp, vp]
     L.srf_marcher_volume_rendering.argtypes = [vp, vp, P(RenderArgs), vp, vp, vp, vp, vp]
     L.srf_compact_rays.argtypes = [vp, u32, vp, vp, vp, vp, vp, vp, vp, vp, vp]

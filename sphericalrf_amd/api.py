@@ -361,7 +361,8 @@ class RayMarcher:
                                                  rgb_activation=K.ACT_LOGISTIC, density_activation=K.ACT_EXPONENTIAL, loss_output=None,
                                                  loss_type=K.LOSS_L2, loss_scale=128.0, density_grid_mean=None, min_optical_thickness=0.01,
                                                  use_grid=True, background_color=(0.0, 0.0, 0.0), color_space=K.COLOR_LINEAR, rng=None,
-                                                 coords=None, compacted_coords=None, dt_stride=1, rgb_ray_out=None):
+                                                 coords=None, compacted_coords=None, dt_stride=1, rgb_ray_out=None, no_alloc=False):
+        """no_alloc: go through the entry point that allocates no device memory (n_rays <= NOALLOC_MAX_RAYS)"""
         a = K.LossArgs()
         a.n_rays, a.n_max_compacted_coords, a.padded_output_width = n_rays, n_max_compacted_coords, padded_output_width
         a.rgb_activation, a.density_activation = int(rgb_activation), int(density_activation)
@@ -372,7 +373,8 @@ class RayMarcher:
         a.rng = (rng or Pcg32()).as_c()
         a.network_output_dtype, a.dloss_dtype = _net_dtype(network_output), _net_dtype(dloss_doutput)
         a.dt_stride = int(dt_stride)
-        K.check(self._L.srf_marcher_volume_rendering_with_loss_and_gradient(
+        entry = self._L.srf_marcher_volume_rendering_with_loss_and_gradient_noalloc if no_alloc else self._L.srf_marcher_volume_rendering_with_loss_and_gradient
+        K.check(entry(
             self._h, C.byref(a), _dev(rays_rgba, torch.float32, 4 * n_rays, "rays_rgba"), _dev(n_rays_counter, torch.int32, 1, "n_rays_counter"),
             _dev(ray_coord_indices, torch.int32, 2 * n_rays, "ray_coord_indices"), _dev(dt, torch.float32, None, "dt"),
             _dev(coords, torch.float32, None, "coords", allow_none=True), _dev(compacted_coords, torch.float32, None, "compacted_coords", allow_none=True),
@@ -402,6 +404,9 @@ class RayMarcher:
         K.check(self._L.srf_marcher_volume_rendering(self._h, sampler._h, C.byref(a), _dev(payloads, torch.uint8, 40 * n_rays, "payloads"),
                                                      _dev(rgba, torch.float32, 4 * n_rays, "rgba"), _dev(coords, torch.float32, 7 * n_rays * n_steps, "coords"),
                                                      _dev(rgbsigma, None, n_rays * n_steps * padded_output_width, "rgbsigma"), _stream()))
+
+
+NOALLOC_MAX_RAYS = 262144   # SRF_NOALLOC_MAX_RAYS
 
 
 # ---- orchestrator kernels (internal/testbed.cu:398-404, 423-477) ---------------------------------

@@ -2,6 +2,7 @@
 // chunked compositing (rendering), and the orchestrator's small kernels
 // (ordered ray compaction, shading, batch roll-over).
 #include "srf_internal.h"
+#include <mutex>
 #include "srf_bodies.h"
 #include "srf_composite_fused.h"
 #include "srf_wave.h"
@@ -72,10 +73,10 @@ struct ChainScratch {
 
 // bytes of device scratch the chain needs for n_rays rays, and where its parts lie (a group makes at most two items)
 struct ChainLayout { size_t off_seg, off_prefix, off_misc, off_words, off_sums, off_items, off_list, off_side, bytes; };
-SRF_HD ChainLayout chain_layout(uint32_t n_rays) {
+SRF_HD constexpr ChainLayout chain_layout(uint32_t n_rays) {
 	const size_t n_groups = ((size_t)n_rays + fused::RAYS - 1) / fused::RAYS;
 	const size_t n_items = 2 * n_groups;
-	ChainLayout L;
+	ChainLayout L = {};
 	L.off_seg = (n_items * 8 + 255) / 256 * 256;
 	L.off_prefix = (L.off_seg + (n_items + 63) / 64 * 8 * SEG_STRIDE + 255) / 256 * 256;
 	L.off_misc = (L.off_prefix + (n_items + 63) / 64 * 8 + 255) / 256 * 256;
@@ -757,6 +758,71 @@ static int launch_stream(const srf_loss_args* a, const LossConst& K, ChainScratc
 
 using namespace srf;
 
+// Argument checks and per-call constants shared by the two training compositing entry points.  *empty: nothing to do.
+static int loss_call_prepare(srf_marcher* m, const srf_loss_args* a, const float* rays_rgba, const uint32_t* n_rays_counter, const uint32_t* ray_coord_indices,
+                             const float* dt, const float* coords, const float* compacted_coords, const uint32_t* n_compacted_coords_counter,
+                             const void* network_output, const void* dloss_doutput, const float* density_grid_mean, LossConst* K_out, bool* empty) {
+	*empty = false;
+	SRF_REQUIRE(m && a, "srf_marcher_volume_rendering_with_loss_and_gradient: NULL argument");
+	if (a->n_rays == 0) { *empty = true; return SRF_OK; }
+	SRF_REQUIRE(rays_rgba && n_rays_counter && ray_coord_indices && dt && n_compacted_coords_counter && network_output && dloss_doutput,
+	            "srf_marcher_volume_rendering_with_loss_and_gradient: NULL buffer");
+	SRF_REQUIRE(!a->use_grid || density_grid_mean, "srf_marcher_volume_rendering_with_loss_and_gradient: use_grid needs density_grid_mean");
+	SRF_REQUIRE((coords == nullptr) == (compacted_coords == nullptr), "srf_marcher_volume_rendering_with_loss_and_gradient: coords and compacted_coords go together");
+	SRF_REQUIRE(a->padded_output_width >= 4, "srf_marcher_volume_rendering_with_loss_and_gradient: padded_output_width must be >= 4");
+	SRF_REQUIRE(a->dt_stride >= 1, "srf_marcher_volume_rendering_with_loss_and_gradient: dt_stride must be >= 1");
+	SRF_REQUIRE(a->loss_type >= SRF_LOSS_L2 && a->loss_type <= SRF_LOSS_RELATIVEL2, "Unknown loss type.");
+	SRF_REQUIRE(a->rgb_activation >= 0 && a->rgb_activation <= 3 && a->density_activation >= 0 && a->density_activation <= 3, "unknown activation");
+	SRF_REQUIRE((a->network_output_dtype | 1) == 1 && (a->dloss_dtype | 1) == 1, "unknown dtype");
+
+	LossConst K;
+	K.n_rays = a->n_rays;
+	K.n_max_compacted = a->n_max_compacted_coords;
+	K.out_width = (uint32_t)a->padded_output_width;
+	K.rgb_act = a->rgb_activation; K.density_act = a->density_activation; K.loss_type = a->loss_type;
+	K.loss_scale = a->loss_scale / (float)a->n_rays;
+	K.min_optical_thickness = a->min_optical_thickness;
+	K.use_grid = a->use_grid;
+	for (int c = 0; c < 3; ++c) K.bg_in[c] = a->background_color[c];
+	if (m->cfg.train_with_random_bg_color) {   // ray_marcher.cu:82-84: one draw shared by all rays
+		Pcg32 r; r.state = a->rng.state; r.inc = a->rng.inc;
+		K.bg_in[0] = pcg_next_float(r); K.bg_in[1] = pcg_next_float(r); K.bg_in[2] = pcg_next_float(r);
+	}
+	loss_const_background(K);
+	K.color_space = a->color_space;
+	K.train_in_linear = m->cfg.train_in_linear_color;
+	K.thr = m->cfg.transmittance_threshold;
+	K.dt_stride = a->dt_stride;
+
+	*K_out = K;
+	return SRF_OK;
+}
+
+// ---- device scratch that exists without any allocation ---------------------------------------
+// The chain's scratch for srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: part of the library's image on every
+// device, found once per device with hipGetSymbolAddress (the array's name means nothing to host code).
+constexpr uint32_t NOALLOC_MAX_RAYS = SRF_NOALLOC_MAX_RAYS;
+constexpr size_t NOALLOC_BYTES = chain_layout(NOALLOC_MAX_RAYS).bytes;
+static __device__ __align__(256) unsigned char g_noalloc_scratch[NOALLOC_BYTES];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static void* g_noalloc_ptr[NOALLOC_MAX_DEVICES];      // per device: where g_noalloc_scratch lies in its memory
+static std::mutex g_noalloc_mutex;
+
+// with the device of the call current
+static int noalloc_scratch(void** out) {
+	int dev = 0;
+	SRF_HIP(hipGetDevice(&dev));
+	if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) SRF_FAIL(SRF_ERR_INVALID, "no-allocation compositing: device index out of range");
+	std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+	if (!g_noalloc_ptr[dev]) {
+		void* p = nullptr;
+		SRF_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_noalloc_scratch)));
+		g_noalloc_ptr[dev] = p;
+	}
+	*out = g_noalloc_ptr[dev];
+	return SRF_OK;
+}
+
 extern "C" {
 
 void srf_marcher_config_default(srf_marcher_config* c) {
@@ -826,40 +892,14 @@ int srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const 
         const float* dt, const float* coords, float* compacted_coords, uint32_t* n_compacted_coords_counter,
         const void* network_output, void* dloss_doutput, float* loss_output,
         const float* density_grid_mean, float* rgb_ray_out, void* stream) {
-	SRF_REQUIRE(m && a, "srf_marcher_volume_rendering_with_loss_and_gradient: NULL argument");
-	if (a->n_rays == 0) return SRF_OK;
-	SRF_REQUIRE(rays_rgba && n_rays_counter && ray_coord_indices && dt && n_compacted_coords_counter && network_output && dloss_doutput,
-	            "srf_marcher_volume_rendering_with_loss_and_gradient: NULL buffer");
-	SRF_REQUIRE(!a->use_grid || density_grid_mean, "srf_marcher_volume_rendering_with_loss_and_gradient: use_grid needs density_grid_mean");
-	SRF_REQUIRE((coords == nullptr) == (compacted_coords == nullptr), "srf_marcher_volume_rendering_with_loss_and_gradient: coords and compacted_coords go together");
-	SRF_REQUIRE(a->padded_output_width >= 4, "srf_marcher_volume_rendering_with_loss_and_gradient: padded_output_width must be >= 4");
-	SRF_REQUIRE(a->dt_stride >= 1, "srf_marcher_volume_rendering_with_loss_and_gradient: dt_stride must be >= 1");
-	SRF_REQUIRE(a->loss_type >= SRF_LOSS_L2 && a->loss_type <= SRF_LOSS_RELATIVEL2, "Unknown loss type.");
-	SRF_REQUIRE(a->rgb_activation >= 0 && a->rgb_activation <= 3 && a->density_activation >= 0 && a->density_activation <= 3, "unknown activation");
-	SRF_REQUIRE((a->network_output_dtype | 1) == 1 && (a->dloss_dtype | 1) == 1, "unknown dtype");
-	hipStream_t st = (hipStream_t)stream;
-
 	LossConst K;
-	K.n_rays = a->n_rays;
-	K.n_max_compacted = a->n_max_compacted_coords;
-	K.out_width = (uint32_t)a->padded_output_width;
-	K.rgb_act = a->rgb_activation; K.density_act = a->density_activation; K.loss_type = a->loss_type;
-	K.loss_scale = a->loss_scale / (float)a->n_rays;
-	K.min_optical_thickness = a->min_optical_thickness;
-	K.use_grid = a->use_grid;
-	for (int c = 0; c < 3; ++c) K.bg_in[c] = a->background_color[c];
-	if (m->cfg.train_with_random_bg_color) {   // ray_marcher.cu:82-84: one draw shared by all rays
-		Pcg32 r; r.state = a->rng.state; r.inc = a->rng.inc;
-		K.bg_in[0] = pcg_next_float(r); K.bg_in[1] = pcg_next_float(r); K.bg_in[2] = pcg_next_float(r);
-	}
-	loss_const_background(K);
-	K.color_space = a->color_space;
-	K.train_in_linear = m->cfg.train_in_linear_color;
-	K.thr = m->cfg.transmittance_threshold;
-	K.dt_stride = a->dt_stride;
-
+	bool empty = false;
+	int rc = loss_call_prepare(m, a, rays_rgba, n_rays_counter, ray_coord_indices, dt, coords, compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput,
+	                           density_grid_mean, &K, &empty);
+	if (rc != SRF_OK || empty) return rc;
+	hipStream_t st = (hipStream_t)stream;
 	const bool hin = a->network_output_dtype == SRF_DTYPE_F16, hout = a->dloss_dtype == SRF_DTYPE_F16;
-	int rc = check_chain_error(m);
+	rc = check_chain_error(m);
 	if (rc != SRF_OK) return rc;
 	// The distortion regulariser's side buffer is only filled by the three-launch implementation, which also serves a marcher
 	// whose chain has failed before, and one created under SRF_COMPOSITE_IMPL=unfused.
@@ -903,6 +943,30 @@ int srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const 
 #undef SRF_BWD
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
+}
+
+int srf_marcher_volume_rendering_with_loss_and_gradient_noalloc(srf_marcher_t* m, const srf_loss_args* a,
+        const float* rays_rgba, const uint32_t* n_rays_counter, uint32_t* ray_coord_indices,
+        const float* dt, const float* coords, float* compacted_coords, uint32_t* n_compacted_coords_counter,
+        const void* network_output, void* dloss_doutput, float* loss_output,
+        const float* density_grid_mean, float* rgb_ray_out, void* stream) {
+	LossConst K;
+	bool empty = false;
+	int rc = loss_call_prepare(m, a, rays_rgba, n_rays_counter, ray_coord_indices, dt, coords, compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput,
+	                           density_grid_mean, &K, &empty);
+	if (rc != SRF_OK || empty) return rc;
+	SRF_REQUIRE(a->n_rays <= NOALLOC_MAX_RAYS, "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: n_rays exceeds SRF_NOALLOC_MAX_RAYS (the scratch built into the library); "
+	            "use srf_marcher_volume_rendering_with_loss_and_gradient");
+	SRF_REQUIRE(m->cfg.regularization_type != SRF_REG_DISTORTION, "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: the distortion regulariser needs buffers that this entry point may not allocate");
+	rc = check_chain_error(m);
+	if (rc != SRF_OK) return rc;
+	SRF_REQUIRE(!m->force_unfused && !m->degraded, "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: this marcher uses the three-launch implementation, which allocates");
+	void* scratch = nullptr;
+	rc = noalloc_scratch(&scratch);
+	if (rc != SRF_OK) return rc;
+	m->chain_error_dev = chain_scratch_at(scratch, a->n_rays, nullptr, 0).error;
+	return launch_stream(a, K, chain_scratch_at(scratch, a->n_rays, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
+	                     compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, (hipStream_t)stream);
 }
 
 int srf_marcher_sync_check(srf_marcher_t* m, void* stream) {

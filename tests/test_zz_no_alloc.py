@@ -1,0 +1,70 @@
+"""The training compositing entry point that allocates nothing
+(srf_marcher_volume_rendering_with_loss_and_gradient_noalloc) against the ordinary entry point: same inputs through
+both, outputs compared bit for bit (integers and float bit patterns), on two calls in a row, the second with a smaller
+input, so that what the first call left in the library's built-in scratch must not matter."""
+import numpy as np
+import pytest
+
+from tests.test_fused_compositing_on_host import layout
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(torch, seed, n_rays, kind):
+    rng = np.random.default_rng(seed)
+    counts, base, total = layout(rng, kind, n_rays)
+    net = rng.random((total, 4)).astype(np.float16)
+    net[:, 3] *= np.float16(3)
+    dt = (rng.random(total) * 0.3 + 0.01).astype(np.float32)
+    tgt = rng.random((n_rays, 4)).astype(np.float32)
+    coords = rng.random((total, 7)).astype(np.float32)
+    idx = np.stack([counts, base], axis=1).astype(np.uint32)
+    cap = int(counts.sum() * 0.9) + 1          # smaller than what the rays keep: the clamp is exercised too
+    dev = lambda x: torch.from_numpy(x).cuda()
+    return dict(n_rays=n_rays, total=total, cap=cap, idx=idx, net=dev(net), dt=dev(dt), tgt=dev(tgt), coords=dev(coords))
+
+
+def _run(torch, api, marcher, w, no_alloc):
+    n_rays, cap = w["n_rays"], w["cap"]
+    idx = torch.from_numpy(w["idx"].view(np.int32)).cuda()
+    dloss = torch.zeros((cap, 4), device="cuda")
+    compacted = torch.zeros((cap, 7), device="cuda")
+    loss, rgb = torch.full((n_rays,), -1.0, device="cuda"), torch.zeros((n_rays, 3), device="cuda")
+    cnt = torch.full((1,), 5, dtype=torch.int32, device="cuda")
+    nrc = torch.full((1,), n_rays - 3, dtype=torch.int32, device="cuda")
+    mean_t = torch.full((1,), 0.001, device="cuda")
+    marcher.volume_rendering_with_loss_and_gradient(n_rays, cap, w["tgt"], nrc, idx, w["dt"], w["net"], dloss, cnt, rgb_activation=api.ACT_LOGISTIC,
+                                                    density_activation=api.ACT_EXPONENTIAL, loss_output=loss, loss_type="SMAPE", density_grid_mean=mean_t,
+                                                    use_grid=True, background_color=(0.2, 0.4, 0.6), coords=w["coords"], compacted_coords=compacted,
+                                                    rgb_ray_out=rgb, no_alloc=no_alloc)
+    marcher.sync_check()
+    return [t.cpu().numpy().view(np.uint32) for t in (cnt, idx, dloss, compacted, loss, rgb)]
+
+
+def test_no_alloc_entry_point_matches_the_ordinary_one_twice_in_a_row(gpu, monkeypatch):
+    torch = gpu
+    from sphericalrf_amd import api
+    monkeypatch.delenv("SRF_COMPOSITE_IMPL", raising=False)
+    cfg = dict(train_with_random_bg_color=True, train_in_linear_color=False)
+    ordinary, no_alloc = api.RayMarcher(cfg), api.RayMarcher(cfg)
+    first = _inputs(torch, 41, 64 * 900 + 17, "gaps")      # several segments of items, holes between rays
+    second = _inputs(torch, 42, 64 * 40 + 5, "split")      # smaller, with groups that are cut into two items
+    for w in (first, second):
+        want = _run(torch, api, ordinary, w, False)
+        got = _run(torch, api, no_alloc, w, True)
+        assert int(want[0][0]) > 5
+        for x, y in zip(want, got):
+            assert np.array_equal(x, y)
+
+
+def test_no_alloc_entry_point_rejects_what_it_cannot_serve(gpu, monkeypatch):
+    torch = gpu
+    from sphericalrf_amd import api, _capi
+    monkeypatch.delenv("SRF_COMPOSITE_IMPL", raising=False)
+    n_rays = api.NOALLOC_MAX_RAYS + 1
+    z = lambda *shape, dtype=torch.float32: torch.zeros(shape, dtype=dtype, device="cuda")
+    args = (n_rays, 16, z(n_rays, 4), z(1, dtype=torch.int32), z(n_rays, 2, dtype=torch.int32), z(16), z(16, 4, dtype=torch.float16), z(16, 4), z(1, dtype=torch.int32))
+    with pytest.raises(_capi.SrfError, match="SRF_NOALLOC_MAX_RAYS"):
+        api.RayMarcher({}).volume_rendering_with_loss_and_gradient(*args, density_grid_mean=z(1), no_alloc=True)
+    with pytest.raises(_capi.SrfError, match="distortion"):
+        api.RayMarcher(dict(regularization_type="Distortion")).volume_rendering_with_loss_and_gradient(64, *args[1:], density_grid_mean=z(1), no_alloc=True)
