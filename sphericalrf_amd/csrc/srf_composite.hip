@@ -975,6 +975,11 @@ int srf_marcher_sync_check(srf_marcher_t* m, void* stream) {
 	if (m->chain_error_dev) {
 		uint32_t flag = 0;
 		SRF_HIP(hipMemcpy(&flag, m->chain_error_dev, 4, hipMemcpyDeviceToHost));
+		if (flag) {      // reported once: the word is cleared, and no later call of this marcher writes it (it has fallen back)
+			const uint32_t zero = 0;
+			SRF_HIP(hipMemcpy(m->chain_error_dev, &zero, 4, hipMemcpyHostToDevice));
+			m->chain_error_dev = nullptr;
+		}
 		if (flag && m->host_error) *m->host_error = 1u;
 		if (flag && !m->host_error) {
 			m->degraded = true;

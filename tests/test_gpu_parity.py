@@ -329,8 +329,10 @@ def test_loss_and_gradient(gpu, orc, hin, hout, variant):
     assert np.array_equal(d_comp.cpu().numpy(), o_comp)
 
 
-@pytest.mark.parametrize("config_id,scale", [(1, 0.5), (3, 0.125)])
+@pytest.mark.parametrize("config_id,scale", [(1, 0.5), (2, 0.25), (2, 1.0), (3, 0.125)])
 def test_render_loop_and_fused_frame(gpu, orc, config_id, scale):
+    """a frame through the fused kernel and through the reference's loop of entry points, against the oracle's frame; (2, 1.0) is
+    workload 2 as it is quoted: 800 x 800 rays over the 128^3 single-cascade grid of a bounded object, 1024 steps"""
     torch = gpu
     from sphericalrf_amd import api, scene
     w, p, grid, bf, mean = helpers.build_scene(orc, config_id, scale)
@@ -384,6 +386,55 @@ def test_render_loop_and_fused_frame(gpu, orc, config_id, scale):
     fb = torch.zeros((res[1], res[0], 4), device="cuda")
     api.shade(int(n_hit.item()), hit_c, hit_p, fb, api.RENDER_SHADE, False)
     assert np.array_equal(fb.cpu().numpy(), want_frame)
+
+
+def test_render_after_the_grid_has_been_updated(gpu, orc):
+    """workload 5's sequence at an eighth of its size: positions drawn from the grid, densities splatted and decayed into it,
+    bitfield rebuilt, and then a frame marched through that bitfield (about half of it occupied, where the blob scenes
+    of the other render tests are sparse); every stage against the oracle"""
+    torch = gpu
+    from sphericalrf_amd import api, scene
+    w = scene.workload(5, 0.125)
+    p = helpers.oracle_params(orc, w["sampler"])
+    s = api.OccupancySampler(w["sampler"])
+    caller, o_caller = api.Pcg32(43), orc.pcg32(43)
+    s.init(1, w["resolution"], w["focal"], (0.5, 0.5), None, None, caller)
+    o_rng = orc.pcg32(orc.next_uint(o_caller), 1)
+    n_total = p.n_total
+    o_grid = np.zeros(n_total, np.float32)
+    rng = np.random.default_rng(5)
+    for step in range(2):
+        n_uni, n_non = (n_total, 0) if step == 0 else (n_total // 2, n_total // 2)
+        n = n_uni + n_non
+        pos, idx = torch.zeros((n, 3), device="cuda"), torch.zeros(n, dtype=torch.int32, device="cuda")
+        s.sample_positions_from_grid(n_uni, n_non, pos, idx)
+        wp1, wi1 = orc.generate_grid_samples(p, n_uni, o_rng, step, o_grid, -0.01)
+        orc.advance(o_rng)
+        wp2, wi2 = orc.generate_grid_samples(p, n_non, o_rng, step, o_grid, p.min_optical_thickness)
+        orc.advance(o_rng)
+        want_idx = np.concatenate([wi1, wi2])
+        assert np.array_equal(u32(idx), want_idx)
+        dens = np.log1p(np.exp(rng.normal(size=(n, 1)))).astype(np.float16)
+        s.update_grid(n, 1, torch.from_numpy(dens).cuda(), idx, api.ACT_NONE)
+        cur = np.zeros(n_total, np.float32)
+        orc.splat_grid_samples(p, want_idx, 1, dens, O.ACT_NONE, cur)
+        orc.ema_grid(cur, p.ema_decay, o_grid)
+        s.update_grid_bitfield()
+    bf, mean = orc.update_grid_bitfield(p, o_grid)
+    assert np.array_equal(s.density_grid_bitfield.cpu().numpy(), bf) and s.density_grid_mean.cpu().numpy()[0] == mean
+    n_cells0 = n_total // p.n_cascades
+    assert 0.2 < np.unpackbits(bf[:n_cells0 // 8]).mean() < 0.8
+    res, f, cam = w["resolution"], w["focal"], w["cameras"][2]
+    table = scene.field_table(4096, 5)
+    table[:, 3] *= 4
+    want_frame, want_ns, _ = orc.render_frame(p, orc.make_field(table, 77), bf, res, f, (0.5, 0.5), cam, transmittance_threshold=1e-4, train_in_linear_colors=True)
+    m = api.RayMarcher(dict(train_in_linear_color=True, transmittance_threshold=1e-4))
+    frame = torch.ones((res[1], res[0], 4), device="cuda")
+    ns = torch.zeros(res[0] * res[1], dtype=torch.int32, device="cuda")
+    s.render_frame_fused(m, api.Field(torch.from_numpy(table).cuda(), 77), res, f, (0.5, 0.5), cam, frame, ns)
+    assert np.array_equal(u32(ns).reshape(res[1], res[0]), want_ns)
+    assert np.array_equal(frame.cpu().numpy(), want_frame)
+    assert (want_frame[..., 3] > 0).mean() > 0.3 and want_ns.sum() > res[0] * res[1]
 
 
 def test_render_modes_and_half_network_output(gpu, orc):
@@ -512,6 +563,53 @@ def test_single_launch_compositing_layouts(gpu, orc, kind, acts, monkeypatch):
         assert np.array_equal(d_dloss.cpu().numpy().view(np.uint32), o_dloss.view(np.uint32))
 
 
+def test_a_look_back_that_gives_up_is_reported_and_the_marcher_falls_back(gpu, orc, monkeypatch):
+    """With no polls allowed, an item of the streaming compositing whose predecessors' counts are not there at its first look
+    gives up (the kernel still drains normally).  The call's counter then reads 0xffffffff, the failure is returned by
+    sync_check, and the marcher's later calls take the three-launch implementation and are right again.  (If every first look
+    succeeds, nothing gives up, and the results must simply be right.)"""
+    monkeypatch.delenv("SRF_COMPOSITE_IMPL", raising=False)
+    torch = gpu
+    from sphericalrf_amd import api, _capi
+    from tests.test_fused_compositing_on_host import layout
+    rng = np.random.default_rng(77)
+    n_rays = 64 * 3000
+    counts, base, total = layout(rng, "short", n_rays)
+    net = helpers.random_network_output(rng, total, np.float16)
+    dt = (rng.random(total) * 0.3 + 0.01).astype(np.float32)
+    tgt = rng.random((n_rays, 4)).astype(np.float32)
+    a = loss_args(n_rays, total, network_output_dtype=O.DTYPE_F16, mean_density=1.0)
+    idx = np.stack([counts, base], axis=1).astype(np.uint32)
+    o_idx, o_dloss = idx.copy(), np.zeros((total, 4), np.float32)
+    o_total = orc.volume_rendering_with_loss_and_gradient(a, tgt, n_rays, o_idx, dt, net, o_dloss)
+    m = api.RayMarcher(dict(train_with_random_bg_color=False, train_in_linear_color=True))
+    m.debug_set_lookback_spin_limit(0)
+    d_tgt, d_dt, d_net = torch.from_numpy(tgt).cuda(), torch.from_numpy(dt).cuda(), torch.from_numpy(net).cuda()
+    nrc, mean_t = torch.full((1,), n_rays, dtype=torch.int32, device="cuda"), torch.ones(1, device="cuda")
+
+    def call():
+        d_idx = torch.from_numpy(idx.view(np.int32)).cuda()
+        d_dloss = torch.zeros((total, 4), device="cuda")
+        cnt = torch.zeros(1, dtype=torch.int32, device="cuda")
+        m.volume_rendering_with_loss_and_gradient(n_rays, total, d_tgt, nrc, d_idx, d_dt, d_net, d_dloss, cnt, rgb_activation=api.ACT_NONE,
+                                                  density_activation=api.ACT_NONE, density_grid_mean=mean_t)
+        return d_idx, d_dloss, cnt
+
+    d_idx, d_dloss, cnt = call()
+    gave_up = False
+    try:
+        m.sync_check()
+    except _capi.SrfError as e:
+        gave_up = True
+        assert "gave up" in str(e)
+        assert int(cnt.item()) & 0xffffffff == 0xffffffff
+    if gave_up:
+        d_idx, d_dloss, cnt = call()      # the three-launch implementation from here on
+        m.sync_check()
+    assert int(cnt.item()) == o_total and np.array_equal(u32(d_idx), o_idx)
+    assert np.array_equal(d_dloss.cpu().numpy().view(np.uint32), o_dloss.view(np.uint32))
+
+
 def test_single_launch_and_three_launch_compositing_agree_at_full_size(gpu, orc, monkeypatch):
     """2^20 rays / ~1.5e7 samples: the streaming implementation and the one-thread-per-ray implementation (selected by the
     environment at creation, or forced by the distortion regulariser) must give identical results, side buffer of the
@@ -590,6 +688,42 @@ def test_full_size_frame_is_the_same_with_and_without_the_empty_space_table(gpu,
     assert torch.equal(out["table"][0].view(torch.int32), out["plain"][0].view(torch.int32))
     assert torch.equal(out["table"][1], out["plain"][1])
     assert int(out["table"][1].sum().item()) > n and float((out["table"][0][..., 3] > 0).float().mean()) > 0.2
+
+
+def test_full_size_frame_after_a_grid_update_is_the_same_with_and_without_the_empty_space_table(gpu, monkeypatch):
+    """Workload 5 in its own order at full size: one update of the 167,772,160-cell grid from drawn positions, bitfield rebuilt
+    (a few tenths of it occupied), then the 1920 x 1080 frame; with the empty-space table and with every step probed"""
+    torch = gpu
+    from sphericalrf_amd import api, scene
+    w = scene.workload(5)
+    res = w["resolution"]
+    n = res[0] * res[1]
+    field = api.Field(torch.from_numpy(scene.field_table(1 << 14, 9)).cuda(), 1234)
+    m = api.RayMarcher(dict(train_in_linear_color=True, transmittance_threshold=1e-4))
+    out = {}
+    for label, env in (("table", "1"), ("plain", "0")):
+        monkeypatch.setenv("SRF_MARCH_SKIP", env)
+        s = api.OccupancySampler(w["sampler"])
+        s.init(1, res, w["focal"], (0.5, 0.5), None, None, api.Pcg32(43))
+        n_total = int(s.n_total_elements)
+        pos, idx = torch.zeros((n_total, 3), device="cuda"), torch.zeros(n_total, dtype=torch.int32, device="cuda")
+        g = torch.Generator(device="cuda")
+        g.manual_seed(48)
+        dens = torch.nn.functional.softplus(torch.randn(n_total, generator=g, device="cuda")).half()
+        s.sample_positions_from_grid(n_total, 0, pos, idx)
+        s.update_grid(n_total, 1, dens, idx, api.ACT_NONE)
+        s.update_grid_bitfield()
+        del pos, idx, dens
+        frame = torch.zeros((res[1], res[0], 4), device="cuda")
+        ns = torch.zeros(n, dtype=torch.int32, device="cuda")
+        s.render_frame_fused(m, field, res, w["focal"], (0.5, 0.5), w["cameras"][3], frame, ns)
+        torch.cuda.synchronize()
+        out[label] = (frame, ns, s.density_grid_bitfield.clone())
+        del s
+    assert torch.equal(out["table"][2], out["plain"][2])
+    assert torch.equal(out["table"][0].view(torch.int32), out["plain"][0].view(torch.int32))
+    assert torch.equal(out["table"][1], out["plain"][1])
+    assert int(out["table"][1].sum().item()) > 4 * n
 
 
 def test_full_size_grid_update_invariants(gpu):
