@@ -15,6 +15,7 @@ the oracle timed on this machine's host cores on a bounded slice of the same wor
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -27,11 +28,20 @@ COMPOSITE_BYTES_PER_SAMPLE = 28  # read fp16 rgb-sigma 8 + fp32 dt 4, write fp32
 COMPOSITE_BYTES_PER_RAY = 36     # read (count, offset) 8 + target 12, write rgb 12 + loss 4
 MARCH_BYTES_PER_SAMPLE = 12      # write t, dt, cell
 MARCH_BYTES_PER_RAY = 32         # read ray 24, write (count, offset) 8
-# HBM bytes per launch of the compositing kernel at this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a plain
-# copy of known size (profiles/training_step_config4_hbm_traffic.txt); counters cannot be read from inside this process
-COMPOSITE_TRAFFIC_BYTES = 454.7e6
+# HBM bytes per launch of the compositing kernel at this workload come from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of the native
+# harness, scaled by a plain copy of known size; counters cannot be read from inside this process, so the figure is read from the
+# committed summary of those runs (None when the file or the line is missing)
+COMPOSITE_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "compositing_config4_hbm_traffic.txt")
 EMA_BYTES_PER_CELL = 12
 BITFIELD_BYTES_PER_CELL = 4.125
+
+
+def composite_traffic_bytes():
+    try:
+        m = re.search(r"^composite_traffic_bytes_per_launch\s*=\s*([0-9.eE+]+)\s*$", open(COMPOSITE_TRAFFIC_PROFILE).read(), re.M)
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def log(*a):
@@ -67,6 +77,8 @@ def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 
     s, grid = build_sampler(torch, api, scene, w)
     log("scene built in %.1f s" % (time.perf_counter() - t0))
     del grid
+    bits = s.density_grid_bitfield
+    occupied_bits = sum(float(torch.bitwise_and(bits >> k, 1).float().mean()) for k in range(8)) / 8
     m = api.RayMarcher(dict(train_with_random_bg_color=False, train_in_linear_color=True, transmittance_threshold=1e-4))
     cams = torch.from_numpy(w["cameras"]).cuda()
     ds = api.Dataset(cams, w["resolution"], w["focal"], (0.5, 0.5))
@@ -132,15 +144,15 @@ def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 
     info = s.info
     return dict(sec_per_step=sec, n_rays=n_rays, n_kept=n_kept, n_samples=n_samples, n_compacted=n_comp, march_ms=march_ms, composite_ms=comp_ms,
                 composite_gbs=comp_bytes / (comp_ms * 1e-3) / 1e9, march_gbs=march_bytes / (march_ms * 1e-3) / 1e9,
-                n_max_steps=int(info.n_max_steps), workload=w, sampler=s)
+                n_max_steps=int(info.n_max_steps), workload=w, sampler=s, occupied_bits=occupied_bits)
 
 
 def cpu_baseline(result, n_rays_sample=1 << 16):
     """the oracle on a slice of the same workload: the first n_rays_sample rays of a batch, march + compositing fwd/bwd"""
     import numpy as np
     from oracle import oracle as O
-    from tests import helpers
-    from tests.test_oracle_composite import loss_args
+    from oracle import support as helpers
+    from oracle.support import loss_args
     orc = O.get()
     w, s = result["workload"], result["sampler"]
     p = helpers.oracle_params(orc, w["sampler"])
@@ -286,14 +298,17 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config 4: training step, 2^20 rays over 200 ring cameras, grid 512x256x256 x 5 cascades, sample cap 2^24, fp16 rgb-sigma in, fp32 gradients out",
-                   "rays": r["n_rays"], "rays_kept": r["n_kept"], "samples": r["n_samples"], "compacted_samples": r["n_compacted"], "max_steps_per_ray": r["n_max_steps"]},
+                   "rays": r["n_rays"], "rays_kept": r["n_kept"], "samples": r["n_samples"], "compacted_samples": r["n_compacted"], "max_steps_per_ray": r["n_max_steps"],
+                   "occupied_bits": r["occupied_bits"],
+                   "scene": "48 + 16 Gaussian blobs thresholded at an absolute level, plus a shell at warped radius 0.9-1.0 over two thirds of the outermost cascade's "
+                            "angular tiles: about 3 % of all bits of the 5 cascades set, which puts the batch's sample total just under the 2^24 cap (no ray is dropped for lack of room)"},
         "rays_per_s": r["n_rays"] / sec,
         "march": {"ms": r["march_ms"], "samples_per_s": r["n_samples"] / (r["march_ms"] * 1e-3), "rays_per_s": r["n_rays"] / (r["march_ms"] * 1e-3),
                   "steps_per_s": r["n_rays"] * r["n_max_steps"] / (r["march_ms"] * 1e-3), "output_gbs": r["march_gbs"], "frac_hbm": r["march_gbs"] / HBM_PEAK_GBS,
                   "bound": "valu issue (serial disparity chain, warp + cell lookup at probed steps), not hbm"},
         "composite": {"ms": r["composite_ms"], "samples_per_s": r["n_samples"] / (r["composite_ms"] * 1e-3), "rays_per_s": r["n_kept"] / (r["composite_ms"] * 1e-3)},
         "roofline": {"kernel": "compositing forward+backward (volume_rendering_with_loss_and_gradient)", "bound": "hbm",
-                     "achieved": r["composite_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": r["composite_gbs"] / HBM_PEAK_GBS, "traffic": COMPOSITE_TRAFFIC_BYTES,
+                     "achieved": r["composite_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": r["composite_gbs"] / HBM_PEAK_GBS, "traffic": composite_traffic_bytes(),
                      "algorithmic_bytes": COMPOSITE_BYTES_PER_SAMPLE * r["n_samples"] + COMPOSITE_BYTES_PER_RAY * r["n_kept"]},
     }
     if not args.no_cpu_baseline:

@@ -429,9 +429,9 @@ struct StreamShared {
 	fused::Plan group_plan;             // plan wave: the group whose rays the item being planned belongs to
 };
 
-// Build flag SRF_STREAM_TIMING: lane 0 of the ray wave and of the first sample wave add up the cycles they spend in
+// Build flag SRF_KERNEL_TIMING: lane 0 of the ray wave and of the first sample wave add up the cycles they spend in
 // the parts of an iteration, into counters after the chain's misc words.
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 #define SRF_T(k) do { if (lane == 0 && wave <= 2) { const unsigned long long now_ = clock64(); t_acc_[k] += now_ - t_prev_; t_prev_ = now_; } } while (0)
 #else
 #define SRF_T(k) ((void)0)
@@ -454,7 +454,7 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 	const uint32_t n_items = *S.n_items;
 	if (blockIdx.x >= n_items) return;
 
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 	unsigned long long t_acc_[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 	unsigned long long t_prev_ = clock64();
 	unsigned long long n_it_ = 0;
@@ -488,15 +488,15 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 		const uint32_t number = number_p;
 		if (number != NO_ITEM) {
 			const uint32_t g = item.x;
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 			{ U2 r_ = rec; asm volatile("" : "+v"(r_.x), "+v"(r_.y)); if (lane == 0 && wave == 1 && t_on_) { const unsigned long long now_ = clock64(); t_acc_[5] += now_ - t_prev_; t_prev_ = now_; } }
 #endif
 			plan_from_records(lane, g, rec, A, sh.group_plan);
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 			if (lane == 0 && wave == 1 && t_on_) { const unsigned long long now_ = clock64(); t_acc_[6] += now_ - t_prev_; t_prev_ = now_; }
 #endif
 			plan_part_lane(lane, sh.group_plan, item_lo(item), item_hi(item), g, out);
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 			if (lane == 0 && wave == 1 && t_on_) { const unsigned long long now_ = clock64(); t_acc_[7] += now_ - t_prev_; t_prev_ = now_; }
 #endif
 		}
@@ -532,7 +532,7 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 		const bool fast = has0 && pl.misc[M_CONTIG] != 0;
 		const bool fast1 = has1 && pl1.misc[M_CONTIG] != 0;
 		const uint32_t ray0 = has0 ? pl.misc[M_GROUP] * RAYS : 0u, lo = has0 ? pl.misc[M_LANE_LO] : 0u, hi = has0 ? pl.misc[M_LANE_HI] : 0u;
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 		if (lane == 0 && wave <= 2) { ++n_it_; t_prev_ = clock64(); t_on_ = true; }
 #endif
 		// ---- first half
@@ -555,7 +555,7 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 				finish_ray(lane, ray0, A, sh.rl, carry, target, lo, hi);
 			}
 		} else {
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 			SRF_T(4);
 #endif
@@ -603,7 +603,7 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 		set_c = set_a;
 		set_a = set_l;
 	}
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 	if (lane == 0 && wave <= 2) {
 		unsigned long long* out = (unsigned long long*)(S.initial + 16) + wave * 12;
 		for (int k = 0; k < 11; ++k) atomicAdd(out + k, t_acc_[k]);
@@ -733,7 +733,7 @@ static int launch_stream(const srf_loss_args* a, const LossConst& K, ChainScratc
 	if (hin && hout) SRF_SLOW_BWD(true, true); else if (hin) SRF_SLOW_BWD(true, false); else if (hout) SRF_SLOW_BWD(false, true); else SRF_SLOW_BWD(false, false);
 #undef SRF_SLOW_BWD
 	SRF_LAUNCH_CHECK();
-#ifdef SRF_STREAM_TIMING
+#ifdef SRF_KERNEL_TIMING
 	{
 		unsigned long long h[36];
 		SRF_HIP(hipStreamSynchronize(st));

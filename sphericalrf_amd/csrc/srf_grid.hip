@@ -396,6 +396,12 @@ int srf_sampler_create(const srf_sampler_config* c, srf_sampler_t** out) {
 	s->skip_dist = nullptr;
 	s->skip_valid = false;
 	{ const char* v = getenv("SRF_MARCH_SKIP"); s->skip_enabled = !(v && v[0] == '0'); }
+	auto tri_state = [](const char* name) { const char* v = getenv(name); return v && v[0] == '0' ? 0 : (v && v[0] == '1' ? 1 : -1); };
+	s->force_splat_sort = tri_state("SRF_SPLAT_SORT");
+	s->force_sample_bits = tri_state("SRF_GRID_SAMPLE_BITS");
+	s->force_sample_by_cell = tri_state("SRF_GRID_SAMPLE_BY_CELL");
+	s->count_probe_budget = COUNT_PROBE_BUDGET;
+	{ const char* v = getenv("SRF_COUNT_PROBE_BUDGET"); if (v && v[0]) s->count_probe_budget = (uint32_t)atoi(v); }
 	hipError_t e = hipSuccess;
 	if (P.use_grid) {
 		e = hipMalloc((void**)&s->density_grid_current, (size_t)s->n_total * sizeof(float));
@@ -505,15 +511,15 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	const uint32_t nc = s->P.n_cells;
 	// With many points to draw, the two comparisons the draws make against the grid (grid > -0.01 for the uniform points,
 	// grid > min_optical_thickness for the others) are tabulated first, one bit per cell: the random lookups then fall on
-	// 1/32 of the memory.  SRF_GRID_SAMPLE_BITS=0|1 forces either way.
+	// 1/32 of the memory.  (force_sample_bits: either way, for the tests.)
 	bool tabulate = (uint64_t)n_uniform + n_nonuniform >= s->n_total / 8;
-	{ const char* v = getenv("SRF_GRID_SAMPLE_BITS"); if (v && v[0] == '0') tabulate = false; else if (v && v[0] == '1') tabulate = true; }
+	if (s->force_sample_bits >= 0) tabulate = s->force_sample_bits != 0;
 	tabulate = tabulate && (uint64_t)n_uniform + n_nonuniform != 0;
 	// Most tries of the second draw fail (few cells are above the threshold), so its cost is the lookups: its points are
-	// dealt to the threads by cell (k_generate_grid_samples_by_cell).  SRF_GRID_SAMPLE_BY_CELL=0|1 forces either way.
+	// dealt to the threads by cell (k_generate_grid_samples_by_cell).  (force_sample_by_cell: either way, for the tests.)
 	const bool can_deal = (nc & (nc - 1u)) == 0u && nc >= 256u && n_nonuniform != 0;
 	bool by_cell = can_deal && n_nonuniform >= 65536u;
-	{ const char* v = getenv("SRF_GRID_SAMPLE_BY_CELL"); if (v && v[0] == '0') by_cell = false; else if (v && v[0] == '1') by_cell = can_deal; }
+	if (s->force_sample_by_cell >= 0) by_cell = s->force_sample_by_cell != 0 && can_deal;
 	// workspace: the two bit tables, then the staging array of the dealt draw (reserved in one go: growing frees)
 	const size_t table_bytes = tabulate ? align_up((size_t)div_up(s->n_total, 32) * 4, 256) : 0;
 	const uint64_t dealt_threads = by_cell ? (uint64_t)div_up(n_nonuniform, nc) * nc : 0;
@@ -529,8 +535,7 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 		SRF_LAUNCH_CHECK();
 		above_a = a; above_b = b;
 	}
-	uint32_t tries = 1;     // looking several candidates up at once (SRF_GRID_SAMPLE_TRIES, up to 4) has made no measurable difference
-	{ const char* v = getenv("SRF_GRID_SAMPLE_TRIES"); if (v && atoi(v) >= 1) tries = (uint32_t)atoi(v); }
+	const uint32_t tries = 1;     // looking several candidates up at once (up to 4) has made no measurable difference
 	if (n_uniform) {
 		hipLaunchKernelGGL(k_generate_grid_samples, dim3(div_up(n_uniform, 256) < 16384u ? div_up(n_uniform, 256) : 16384u), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
 		                   (const float*)s->density_grid, -0.01f, grid_positions, grid_indices, above_a, 1u);   // nearly every first try passes
@@ -571,7 +576,7 @@ int srf_sampler_update_grid(srf_sampler_t* s, uint32_t n_total_positions, uint32
 	SRF_REQUIRE(density_activation >= SRF_ACT_NONE && density_activation <= SRF_ACT_EXPONENTIAL, "srf_sampler_update_grid: unknown activation");
 	hipStream_t st = (hipStream_t)stream;
 	bool sorted_splat = n_total_positions >= SPLAT_SORT_MIN;
-	{ const char* v = getenv("SRF_SPLAT_SORT"); if (v && v[0] == '0') sorted_splat = false; else if (v && v[0] == '1') sorted_splat = n_total_positions != 0; }
+	if (s->force_splat_sort >= 0) sorted_splat = s->force_splat_sort != 0 && n_total_positions != 0;
 	int rc = sorted_splat ? SRF_OK : fill_u32(s->density_grid_current, s->n_total, 0u, st);
 	if (rc != SRF_OK) return rc;
 	if (sorted_splat) {

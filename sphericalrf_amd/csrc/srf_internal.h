@@ -27,6 +27,8 @@ struct Workspace {
 	void release();
 };
 
+constexpr uint32_t COUNT_PROBE_BUDGET = 192;   // lookups after which the counting march parks a ray for the wide march
+
 SRF_HD uint32_t div_up(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 inline size_t align_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
 
@@ -53,6 +55,11 @@ struct srf_sampler {
 	uint16_t* skip_dist;     // empty-space radii per block (srf_skip.h); rebuilt with the bitfield
 	bool     skip_valid;    // skip_dist matches the bitfield
 	bool     skip_enabled;  // SRF_MARCH_SKIP=0 in the environment at creation switches the table off
+	// Switches the tests use to run both sides of a size-dependent choice on small inputs; read from the environment once, when the
+	// sampler is created (-1: the library chooses): SRF_SPLAT_SORT, SRF_GRID_SAMPLE_BITS, SRF_GRID_SAMPLE_BY_CELL = 0|1;
+	// SRF_COUNT_PROBE_BUDGET = lookups after which the counting march parks a ray (0: never)
+	int      force_splat_sort, force_sample_bits, force_sample_by_cell;
+	uint32_t count_probe_budget;
 	srf::Workspace ws;
 };
 

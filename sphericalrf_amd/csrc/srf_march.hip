@@ -54,7 +54,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(SRF_COU
                                                                                                                     const uint32_t* __restrict__ order, unsigned long long* timing) {
 	const uint32_t lane = threadIdx.x;
 	uint32_t next = blockIdx.x * rays_per_wave;
-#ifdef SRF_COUNT_TIMING
+#ifdef SRF_KERNEL_TIMING
 	// per phase (step, probe, begin): cycles, rounds, lanes that took part
 	unsigned long long t_acc_[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 	unsigned long long t_prev_ = clock64();
@@ -91,7 +91,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(SRF_COU
 			SRF_COUNT_STAMP(2, n_idle);
 		}
 	}
-#ifdef SRF_COUNT_TIMING
+#ifdef SRF_KERNEL_TIMING
 	if (lane == 0) {
 		for (int k = 0; k < 9; ++k) atomicAdd(&timing[(blockIdx.x & 1023u) * 16 + k], t_acc_[k]);
 		atomicAdd(&timing[(blockIdx.x & 1023u) * 16 + 9], clock64() - t_first_);
@@ -308,12 +308,11 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 	uint32_t log_words = s->P.use_grid ? (s->P.n_max_steps + 64 + 31) / 32 : 0;
 	if (log_words > LOG_MAX_WORDS) log_words = LOG_MAX_WORDS;
 	const size_t off_log = align_up(off_scan + scan_scratch_bytes(n_rays), 256);
-	// marching order: chunks of rays sorted by (image, pixel tile); SRF_MARCH_SORT=0 keeps index order
-	static const bool sort_rays = [] { const char* v = getenv("SRF_MARCH_SORT"); return !(v && v[0] == '0'); }();
+	// marching order: chunks of rays sorted by (image, pixel tile)
+	constexpr bool sort_rays = true;
 	const size_t off_order = align_up(off_log + (size_t)log_words * n * 8, 256);
-	// rays that exhaust their probe budget are parked and finished by the wide march (SRF_COUNT_PROBE_BUDGET, 0 = never)
-	uint32_t probe_budget = 192;
-	{ const char* v = getenv("SRF_COUNT_PROBE_BUDGET"); if (v && v[0]) probe_budget = (uint32_t)atoi(v); }
+	// rays that exhaust their probe budget are parked and finished by the wide march (0 = never)
+	const uint32_t probe_budget = s->count_probe_budget;
 	const uint32_t parked_capacity = probe_budget ? (n_rays / 8u > 4096u ? n_rays / 8u : 4096u) : 0u;
 	const size_t off_parked = align_up(off_order + (sort_rays ? n * 4 : 0), 256);
 	const size_t off_parked_count = align_up(off_parked + (size_t)parked_capacity * sizeof(ParkedRay), 256);
@@ -349,13 +348,9 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 	ca.parked_count = (uint32_t*)(w + off_parked_count);
 	if (probe_budget) hipLaunchKernelGGL(k_zero_word, dim3(1), dim3(1), 0, st, ca.parked_count);
 	// rays per wavefront: enough for lanes that finish early to pick up more work, few enough for several wavefronts per SIMD
-	uint32_t rays_per_wave = 64;
-	{ const char* v = getenv("SRF_COUNT_RAYS_PER_WAVE"); if (v && atoi(v) >= 64) rays_per_wave = (uint32_t)atoi(v); }
-	uint32_t probe_quorum = 64, begin_quorum = 32;
-	{ const char* v = getenv("SRF_COUNT_PROBE_QUORUM"); if (v && atoi(v) >= 1) probe_quorum = (uint32_t)atoi(v); }
-	{ const char* v = getenv("SRF_COUNT_BEGIN_QUORUM"); if (v && atoi(v) >= 1) begin_quorum = (uint32_t)atoi(v); }
-	uint32_t probe_ratio = 8;
-	{ const char* v = getenv("SRF_COUNT_PROBE_RATIO"); if (v && atoi(v) >= 1) probe_ratio = (uint32_t)atoi(v); }
+	// (settled by measurement on the 2^20-ray training batch: one ray a lane; a probe round once every lane waits for one or the stepping
+	// lanes are outnumbered 8 to 1; new rays are begun 32 at a time)
+	constexpr uint32_t rays_per_wave = 64, probe_quorum = 64, begin_quorum = 32, probe_ratio = 8;
 	const uint32_t* order = nullptr;
 	if (sort_rays) {
 		uint32_t* order_out = (uint32_t*)(w + off_order);
@@ -364,13 +359,13 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 		order = order_out;
 	}
 	unsigned long long* timing = nullptr;
-#ifdef SRF_COUNT_TIMING
+#ifdef SRF_KERNEL_TIMING
 	static unsigned long long* timing_buf = nullptr;
 	if (!timing_buf) { SRF_HIP(hipMalloc((void**)&timing_buf, (1024 * 16 + 192) * 8)); SRF_HIP(hipMemset(timing_buf, 0, (1024 * 16 + 192) * 8)); }
 	timing = timing_buf;
 #endif
 	hipLaunchKernelGGL(k_train_count, dim3(div_up(n_rays, rays_per_wave)), dim3(64), 0, st, s->P, ca, rays_per_wave, probe_quorum, begin_quorum, probe_ratio, order, timing);
-#ifdef SRF_COUNT_TIMING
+#ifdef SRF_KERNEL_TIMING
 	{
 		static unsigned long long hs[1024 * 16 + 192];
 		unsigned long long h[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};

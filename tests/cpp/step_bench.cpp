@@ -1,7 +1,7 @@
 // Torch-free driver of one training step (march + compositing forward/backward) through include/srf_hip.hpp,
 // for timing and for profiler runs (a process that holds nothing but this library's kernels and a few fill kernels).
 //
-//   step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite] [--verify]
+//   step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite] [--verify] [--copy-check]
 //
 // The workload file (written by sphericalrf_amd.scene.write_workload_file) holds the sampler configuration, the
 // cameras, the occupancy bitfield and a table of (r, g, b, sigma) rows; per-sample network output and per-ray targets
@@ -10,6 +10,8 @@
 // same buffer sizing, the network replaced by the table.
 // Prints one JSON line: sizes, milliseconds per entry point (HIP events on the stream the calls are enqueued on).
 // --verify also runs the one-thread-per-ray compositing implementation on the same inputs and compares every output bit.
+// --copy-check ends with three launches of a plain copy of 256 MiB (k_plain_copy reads 2^28 bytes and writes 2^28 bytes), so that
+// a profiler's HBM byte counters of the same run can be scaled by what they read for a kernel of known traffic.
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <cstdio>
@@ -25,6 +27,11 @@
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
 	x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
 	return x;
+}
+
+// reads n 16-byte words and writes them elsewhere: a kernel whose HBM traffic is known
+__global__ void __launch_bounds__(256) k_plain_copy(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n) {
+	for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
 }
 
 // float grid holding 1 where the bitfield has a bit and 0 elsewhere
@@ -95,9 +102,9 @@ struct Timer {
 };
 
 int main(int argc, char** argv) {
-	if (argc < 2) { std::fprintf(stderr, "usage: step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite] [--verify]\n"); return 2; }
+	if (argc < 2) { std::fprintf(stderr, "usage: step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite] [--verify] [--copy-check]\n"); return 2; }
 	uint32_t steps = 10, warmup = 2, n_rays = 1u << 20, cap = 1u << 24;
-	bool verify = false;
+	bool verify = false, copy_check = false;
 	std::string only;
 	for (int i = 2; i < argc; ++i) {
 		const std::string a = argv[i];
@@ -108,6 +115,7 @@ int main(int argc, char** argv) {
 		else if (a == "--cap") cap = (uint32_t)std::atoi(next());
 		else if (a == "--only") only = next();
 		else if (a == "--verify") verify = true;
+		else if (a == "--copy-check") copy_check = true;
 		else { std::fprintf(stderr, "unknown option %s\n", a.c_str()); return 2; }
 	}
 	const Workload w = load_workload(argv[1]);
@@ -246,6 +254,16 @@ int main(int argc, char** argv) {
 			const bool same = after == n_compacted && std::memcmp(a.data(), b.data(), n_out * 4) == 0 && std::memcmp(la_.data(), lb_.data(), (size_t)n_rays * 4) == 0 &&
 			                  std::memcmp(ca.data(), cb.data(), (size_t)n_rays * 12) == 0 && std::memcmp(ia.data(), ib.data(), (size_t)n_rays * 8) == 0;
 			verify_rc = same ? 0 : 1;
+		}
+
+		if (copy_check) {
+			const size_t n_words = (size_t)1 << 24;     // 2^24 x 16 B = 256 MiB each way
+			uint4* src = dev_alloc<uint4>(n_words);
+			uint4* dst = dev_alloc<uint4>(n_words);
+			HIP_OK(hipMemset(src, 1, n_words * 16));
+			for (int k = 0; k < 3; ++k) hipLaunchKernelGGL(k_plain_copy, dim3(4096), dim3(256), 0, st, (const uint4*)src, dst, n_words);
+			HIP_OK(hipStreamSynchronize(st));
+			HIP_OK(hipFree(src)); HIP_OK(hipFree(dst));
 		}
 
 		const double comp_bytes = 28.0 * n_samples + 36.0 * n_kept;

@@ -242,9 +242,6 @@ def test_full_size_march_is_the_same_whatever_the_probe_budget(gpu, monkeypatch)
     centres, sigmas = scene.blob_set(**w["blobs"])
     grid = scene.density_grid_from_blobs(w["sampler"]["grid_size"], w["sampler"]["num_cascades"], centres, sigmas, w["occupancy"], w["shell"], w["seed"], device="cuda")
     ds = api.Dataset(torch.from_numpy(w["cameras"]).cuda(), w["resolution"], w["focal"], (0.5, 0.5))
-    s = api.OccupancySampler(w["sampler"])
-    s.set_density_grid(grid)
-    s.update_grid_bitfield()
     n_rays, cap = 1 << 17, 1 << 22
     out = {}
     for budget in (None, "0", "3", "40"):
@@ -252,6 +249,9 @@ def test_full_size_march_is_the_same_whatever_the_probe_budget(gpu, monkeypatch)
             monkeypatch.delenv("SRF_COUNT_PROBE_BUDGET", raising=False)
         else:
             monkeypatch.setenv("SRF_COUNT_PROBE_BUDGET", budget)
+        s = api.OccupancySampler(w["sampler"])      # the budget is read when a sampler is created
+        s.set_density_grid(grid)
+        s.update_grid_bitfield()
         rays = torch.zeros((n_rays, 6), device="cuda")
         ns = torch.zeros((n_rays, 2), dtype=torch.int32, device="cuda")
         rgba = torch.zeros((n_rays, 4), device="cuda")

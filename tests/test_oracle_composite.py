@@ -6,25 +6,8 @@ import pytest
 
 from oracle import oracle as O
 from sphericalrf_amd import scene
+from oracle.support import loss_args  # noqa: F401  (other test modules import it from here)
 from tests import helpers
-
-
-def loss_args(n_rays, cap, **kw):
-    a = O.LossArgs()
-    a.n_rays, a.n_max_compacted_coords, a.padded_output_width = n_rays, cap, 4
-    a.rgb_activation, a.density_activation = O.ACT_NONE, O.ACT_NONE
-    a.loss_type, a.loss_scale = O.LOSS_L2, 128.0
-    a.regularization_type = O.REG_NONE
-    a.mean_density, a.min_optical_thickness, a.use_grid = 1.0, 0.01, 1
-    a.background_color = (O.f32 * 3)(0, 0, 0)
-    a.color_space = O.COLOR_LINEAR
-    a.train_with_random_bg_color, a.train_in_linear_color = 0, 1
-    a.transmittance_threshold = 1e-4
-    a.rng = O.Pcg32(1, 1)
-    a.network_output_dtype, a.dloss_dtype, a.dt_stride = O.DTYPE_F32, O.DTYPE_F32, 1
-    for k, v in kw.items():
-        setattr(a, k, v)
-    return a
 
 
 def run(orc, a, counts, net, dt, targets, n_active=None, counter0=0):
