@@ -118,6 +118,11 @@ __device__ inline void status_store(unsigned long long* p, uint32_t flag, uint32
 	__hip_atomic_store(p, ((unsigned long long)flag << 32) | value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// a segment's prefix word only ever goes up: nothing (0) -> prefix (flag 2) -> an item gave up (flag 3), whoever writes last
+__device__ inline void status_raise(unsigned long long* p, uint32_t flag, uint32_t value) {
+	(void)__hip_atomic_fetch_max(p, ((unsigned long long)flag << 32) | value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // An item's count, visible to every item after it (one lane): its own status word, and its share of its segment's running total.
 __device__ inline void chain_publish(const ChainScratch& S, uint32_t i, uint32_t total) {
 	if (lane_id() == 0) {
@@ -196,7 +201,7 @@ __device__ inline uint32_t chain_resolve(const ChainScratch& S, uint32_t i, uint
 	if (failed) {
 		if (lane == 0) {
 			status_store(&S.item_status[i], 3u, 0u);
-			status_store(&S.seg_prefix[seg], 3u, 0u);
+			status_raise(&S.seg_prefix[seg], 3u, 0u);
 			atomicExch(S.error, 1u);
 			if (S.host_error) __hip_atomic_store(S.host_error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 		}
@@ -204,8 +209,8 @@ __device__ inline uint32_t chain_resolve(const ChainScratch& S, uint32_t i, uint
 	}
 	// shortcuts for later look-backs: the prefix up to the end of the segment before this one, and up to the end of this one
 	if (lane == 0) {
-		if (j == 0 && seg != 0) status_store(&S.seg_prefix[seg - 1], 2u, before);
-		if (j == WAVE - 1) status_store(&S.seg_prefix[seg], 2u, before + within + total);
+		if (j == 0 && seg != 0) status_raise(&S.seg_prefix[seg - 1], 2u, before);
+		if (j == WAVE - 1) status_raise(&S.seg_prefix[seg], 2u, before + within + total);
 	}
 	return before + within;
 }
@@ -367,7 +372,7 @@ __global__ void __launch_bounds__(fused::WideGeometry::THREADS) k_slow_groups(fu
 			if (!BACKWARD) {
 				if (live) S.side[ray0 + lane] = sh.rl.rnf[lane];
 			} else {
-				if (wave == 0) commit_ray(lane, ray0, live ? S.side[ray0 + lane] : 0u, A, sh.rl);
+				if (wave == 0) commit_ray(lane, ray0, live ? S.side[ray0 + lane] : 0u, A, sh.rl, pl);
 				group_sync();
 				if (wave == 0) reset_carry(lane, pl, c);
 				for (uint32_t win = 0; win < n_win; ++win) {
@@ -545,7 +550,7 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 				const uint32_t prefix = chain_resolve(S, i_0, total_cur, peek);
 				SRF_T(6);
 				const uint32_t cbase = prefix == CHAIN_FAILED ? CHAIN_FAILED : prefix + incl_cur - n_cur;
-				if (fast) commit_ray(lane, ray0, cbase, A, sh.rl, lo, hi, false);
+				if (fast) commit_ray(lane, ray0, cbase, A, sh.rl, pl, lo, hi, false);
 				else if (ray0 + lane < A.n_active) S.side[ray0 + lane] = cbase;
 				if (i_0 == n_items - 1 && lane == 0) *compacted_counter = prefix == CHAIN_FAILED ? CHAIN_FAILED : prefix + total_cur;
 			}
@@ -576,19 +581,20 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 				total_cur = (uint32_t)__shfl((int)incl_cur, WAVE - 1, WAVE);
 				chain_publish(S, i_1, total_cur);
 				SRF_T(7);
-				if (fast1) chain_counted<G>(lane, n_cur, wave_max_u32(n_cur), w1, sh.rl, pl1, carry);
+				if (fast1) chain_counted<G, false>(lane, n_cur, wave_max_u32(n_cur), w1, sh.rl, pl1, carry);
 				peek = chain_peek(S, i_1);                            // needed in the next first half; the items before this one have published by now unless their workgroups lag
 				SRF_T(4);
 			}
 		} else if (plan_wave) {
 			// the plan first: it waits for records requested an iteration ago, and that wait must not include anything younger (see above)
 			plan_next(pl3);
+			if (fast1) mark_owners<G>(lane, wave_max_u32(pl1.rn[lane]), w1, pl1);     // which ray each sample of item it + 1 belongs to, for its phase C
 			SRF_T(4);
 			if (has1) {
 				const uint32_t ray1 = pl1.misc[M_GROUP] * RAYS;
 				if (ray1 + lane < A.n_active) target = *(const Float4*)(A.rays_rgba + 4 * (size_t)(ray1 + lane));
 			}
-			if (fast) commit_loss(lane, ray0, A, sh.rl, lo, hi);
+			if (fast) commit_loss(lane, ray0, A, sh.rl, pl, lo, hi);
 			if (fast) coords_copy_single<G>(lane, A, w, sh.rl, pl);
 		} else {
 			if (has2 && pl2.misc[M_CONTIG] != 0) phase_a_load_single<G, HALF_IN>(st_id, A, pl2, set_l);

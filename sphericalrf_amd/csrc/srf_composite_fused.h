@@ -82,9 +82,9 @@ constexpr uint32_t NO_ITEM = 0xffffffffu;
 // per ray, read by phase C
 struct alignas(16) RayOut {
 	float g[3];         // d loss / d colour
-	uint32_t cbase;     // compacted offset
+	uint32_t obase;     // compacted offset of the ray minus the position of its first sample in the group: a kept sample at position s lands at obase + s
 	float c[3];         // composited colour
-	uint32_t n_kept;    // samples kept after the compacted-capacity clamp
+	uint32_t s_end;     // position in the group after the ray's last kept sample (kept: after the compacted-capacity clamp)
 };
 
 // where a group's rays lie in the sample buffer
@@ -159,7 +159,7 @@ SRF_HD bool item_listed(U2 item) { return (item.y >> 16) != 0; }
 constexpr uint32_t NO_OWNER = 0xffu;
 
 // one window of samples in LDS
-//   S      phase A: {alpha, r, g, b}; after the chain: {T after the sample, colour prefix r, g, b}
+//   S      phase A: {alpha, r, g, b}; after the chain: {T before the sample, colour sum r, g, b including it}
 //   owner  which ray's chain consumed the sample (NO_OWNER: none), written by the chain, read by phase C
 constexpr uint32_t CHAIN_LOOKAHEAD = 8;   // records the ray loops may read past a ray's last sample (they are not used)
 template <class G>
@@ -172,7 +172,6 @@ struct Window {
 struct RayLds {
 	RayOut out[RAYS];
 	uint32_t rnf[RAYS];         // samples consumed by the forward pass (early termination)
-	float Tin[RAYS];            // transmittance of the ray at the start of the current window
 	float loss[RAYS];           // loss of the ray, parked until the clamp is known
 	Float4 carry[RAYS];         // transmittance and colour sum the chain left (for a kernel whose chain and finish run on different waves)
 };
@@ -366,11 +365,15 @@ SRF_HD uint32_t count_lane(uint32_t lane, uint32_t n_max, const Args& A, const W
 		float a[COUNT_UNROLL];
 		#pragma unroll
 		for (uint32_t u = 0; u < COUNT_UNROLL; ++u) a[u] = S[base + k + u < last ? base + k + u : last].x;
+		// only the products depend on one another: the first step at which the test holds is the smallest such step
+		uint32_t first = 0xffffffffu;
 		#pragma unroll
 		for (uint32_t u = 0; u < COUNT_UNROLL; ++u) {
-			cnt = (T < thr && k + u < cnt) ? k + u : cnt;
+			const uint32_t here = T < thr ? k + u : 0xffffffffu;
+			first = here < first ? here : first;
 			T *= (1.f - a[u]);
 		}
+		cnt = first < cnt ? first : cnt;
 	}
 	return cnt;
 }
@@ -379,23 +382,38 @@ SRF_HD uint32_t count_lane(uint32_t lane, uint32_t n_max, const Args& A, const W
 // The reference's loop over the n_fwd samples count_lane found: no termination test is left in it.  Every lane runs
 // n_max steps (the largest n_fwd among the lanes that run together); steps past a lane's n_fwd change nothing.
 // The steps [k_lo, k_hi) of that loop (k_lo a multiple of CHAIN_UNROLL; the lane's ray is carried in c from one stretch to the next).
-template <class G>
+// MARK_OWNER = false: the samples' owner marks are written elsewhere (mark_owners)
+template <class G, bool MARK_OWNER = true>
 SRF_HD void chain_counted_steps(uint32_t lane, uint32_t n_fwd, uint32_t k_lo, uint32_t k_hi, Window<G>& w, const Plan& pl, RayCarry& c) {
 	const uint32_t base = pl.rbase[lane];
+	const uint32_t last = G::WIN + CHAIN_LOOKAHEAD - 1;
 	float T = c.T, r = c.Cr, g = c.Cg, b = c.Cb;
 	for (uint32_t k = k_lo; k < k_hi; k += CHAIN_UNROLL) {
 		Float4 v[CHAIN_UNROLL];
 		#pragma unroll
-		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) v[u] = w.S[base + k + u < G::WIN + CHAIN_LOOKAHEAD - 1 ? base + k + u : G::WIN + CHAIN_LOOKAHEAD - 1];
+		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) v[u] = w.S[base + k + u < last ? base + k + u : last];
+		// A step past the ray's count runs on an all-zero record (what was read there may be anything, not-a-number included), which
+		// leaves T (times 1) and the colour sums (plus 0) as they are, so the stretch needs no branches; written so that only T's
+		// products and each colour's sums depend on one another.
+		float a[CHAIN_UNROLL], Tb[CHAIN_UNROLL], wgt[CHAIN_UNROLL];
+		Float4 out[CHAIN_UNROLL];
+		#pragma unroll
+		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) {
+			if (!(k + u < n_fwd)) v[u] = mk4(0.f, 0.f, 0.f, 0.f);
+			a[u] = v[u].x;
+		}
+		#pragma unroll
+		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) { Tb[u] = T; wgt[u] = a[u] * T; T *= (1.f - a[u]); }
+		#pragma unroll
+		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) {
+			r += wgt[u] * v[u].y; g += wgt[u] * v[u].z; b += wgt[u] * v[u].w;
+			out[u] = mk4(Tb[u], r, g, b);
+		}
 		#pragma unroll
 		for (uint32_t u = 0; u < CHAIN_UNROLL; ++u) {
 			if (k + u < n_fwd) {
-				const float alpha = v[u].x;
-				const float weight = alpha * T;
-				r += weight * v[u].y; g += weight * v[u].z; b += weight * v[u].w;
-				T *= (1.f - alpha);
-				w.S[base + k + u] = mk4(T, r, g, b);
-				w.owner[base + k + u] = (uint8_t)lane;
+				w.S[base + k + u] = out[u];
+				if (MARK_OWNER) w.owner[base + k + u] = (uint8_t)lane;
 			}
 		}
 	}
@@ -407,11 +425,20 @@ SRF_HD void chain_counted_end(uint32_t lane, uint32_t n_fwd, RayLds& rl, const P
 	rl.rnf[lane] = n_fwd;
 	rl.carry[lane] = mk4(c.T, c.Cr, c.Cg, c.Cb);
 }
-template <class G>
+template <class G, bool MARK_OWNER = true>
 SRF_HD void chain_counted(uint32_t lane, uint32_t n_fwd, uint32_t n_max, Window<G>& w, RayLds& rl, const Plan& pl, RayCarry& c) {
 	chain_counted_begin(c);
-	chain_counted_steps<G>(lane, n_fwd, 0, n_max, w, pl, c);
+	chain_counted_steps<G, MARK_OWNER>(lane, n_fwd, 0, n_max, w, pl, c);
 	chain_counted_end(lane, n_fwd, rl, pl, c);
+}
+
+// Owner marks of a one-window plan, lane <-> ray: every sample in a ray's range is marked with the ray, whether or not the
+// chain will consume it (phase C tells by the ray's count); n_max: the largest range among the lanes that run together.
+// After phase A, which marks every sample as nobody's.
+template <class G>
+SRF_HD void mark_owners(uint32_t lane, uint32_t n_max, Window<G>& w, const Plan& pl) {
+	const uint32_t base = pl.rbase[lane], n = pl.rn[lane];
+	for (uint32_t k = 0; k < n_max; ++k) if (k < n) w.owner[base + k] = (uint8_t)lane;
 }
 
 // where chain_counted left the lane's ray, read back by another wave
@@ -423,10 +450,9 @@ SRF_HD void carry_from_lds(uint32_t lane, const RayLds& rl, const Plan& pl, RayC
 
 // ---- chain over one window of a longer group: lane <-> ray (ray_marcher.cu:63-79; the same loop again at :171-182) ----
 // Walks the ray's samples inside this window in order: early-termination test, weight,
-// colour sum, transmittance; leaves {T after the sample, colour sum including it} in place.
+// colour sum, transmittance; leaves {T before the sample, colour sum including it} in place.
 template <class G>
 SRF_HD void chain(uint32_t lane, uint32_t win, const Args& A, Window<G>& w, RayLds& rl, const Plan& pl, RayCarry& c) {
-	rl.Tin[lane] = c.T;
 	const uint32_t base = pl.rbase[lane];
 	const uint32_t win_lo = win * G::WIN;
 	// samples of this ray that lie in the window: k in [c.k, k_end)
@@ -449,8 +475,8 @@ SRF_HD void chain(uint32_t lane, uint32_t win, const Args& A, Window<G>& w, RayL
 			const float alpha = v[u].x;
 			const float weight = alpha * T;
 			r += weight * v[u].y; g += weight * v[u].z; b += weight * v[u].w;
-			T *= (1.f - alpha);
 			w.S[base + k - win_lo] = mk4(T, r, g, b);
+			T *= (1.f - alpha);
 			w.owner[base + k - win_lo] = (uint8_t)lane;
 			++k;
 		}
@@ -482,24 +508,25 @@ SRF_HD void finish_ray(uint32_t lane, uint32_t ray0, const Args& A, RayLds& rl, 
 
 // after the ordered offset of the ray is known (ray_marcher.cu:116-131)
 // write_loss = false: the ray's loss is written later, by commit_loss (a kernel whose finish may still be running on another wave)
-SRF_HD void commit_ray(uint32_t lane, uint32_t ray0, uint32_t cbase, const Args& A, RayLds& rl, uint32_t lane_lo = 0, uint32_t lane_hi = RAYS, bool write_loss = true) {
+SRF_HD void commit_ray(uint32_t lane, uint32_t ray0, uint32_t cbase, const Args& A, RayLds& rl, const Plan& pl, uint32_t lane_lo = 0, uint32_t lane_hi = RAYS, bool write_loss = true) {
 	const uint32_t i = ray0 + lane;
 	RayOut& o = rl.out[lane];
-	o.cbase = cbase;
-	if (i >= A.n_active || lane < lane_lo || lane >= lane_hi) { o.n_kept = 0; return; }
+	const uint32_t first = pl.rbase[lane];
+	o.obase = cbase - first;
+	if (i >= A.n_active || lane < lane_lo || lane >= lane_hi) { o.s_end = first; return; }
 	uint32_t n = rl.rnf[lane];
 	const uint32_t room = A.K.n_max_compacted - (A.K.n_max_compacted < cbase ? A.K.n_max_compacted : cbase);
 	n = room < n ? room : n;
-	o.n_kept = n;
+	o.s_end = first + n;
 	A.ray_coord_indices[2 * (size_t)i] = n;
 	A.ray_coord_indices[2 * (size_t)i + 1] = cbase;
 	if (write_loss && n != 0 && A.loss_output) A.loss_output[i] = rl.loss[lane];
 }
 
-SRF_HD void commit_loss(uint32_t lane, uint32_t ray0, const Args& A, const RayLds& rl, uint32_t lane_lo = 0, uint32_t lane_hi = RAYS) {
+SRF_HD void commit_loss(uint32_t lane, uint32_t ray0, const Args& A, const RayLds& rl, const Plan& pl, uint32_t lane_lo = 0, uint32_t lane_hi = RAYS) {
 	const uint32_t i = ray0 + lane;
 	if (i >= A.n_active || lane < lane_lo || lane >= lane_hi) return;
-	if (rl.out[lane].n_kept != 0 && A.loss_output) A.loss_output[i] = rl.loss[lane];
+	if (rl.out[lane].s_end != pl.rbase[lane] && A.loss_output) A.loss_output[i] = rl.loss[lane];
 }
 
 // ---- phase C: thread <-> sample (ray_marcher.cu:171-201) ---------------------------------
@@ -520,17 +547,17 @@ SRF_HD void phase_c(uint32_t tid, uint32_t win, const Args& A, const Window<G>& 
 		if (win * G::WIN + q >= total) continue;
 		const uint32_t r = w.owner[q];
 		if (r >= RAYS) continue;
-		const uint32_t k = win * G::WIN + q - pl.rbase[r];
-		const Float4 og = *(const Float4*)&rl.out[r].g[0];      // g.xyz, cbase
-		const Float4 oc = *(const Float4*)&rl.out[r].c[0];      // c.xyz, n_kept
-		if (k >= srf_f2u(oc.w)) continue;
-		const Float4 after = w.S[q];                             // T after the sample, colour prefix including it
-		const float T_before = (k == 0) ? 1.f : (q == 0 ? rl.Tin[r] : w.S[q - 1].x);
+		const uint32_t srel = win * G::WIN + q;                  // position in the group
+		const Float4 og = *(const Float4*)&rl.out[r].g[0];      // g.xyz, obase
+		const Float4 oc = *(const Float4*)&rl.out[r].c[0];      // c.xyz, s_end
+		if (srel >= srf_f2u(oc.w)) continue;
+		const Float4 after = w.S[q];                             // T before the sample, colour sum including it
+		const float T_before = after.x;
 		float v[4];
 		unpack_raw<HALF_IN>(st.raw[j], v);
 		const float cr = act_rgb(v[0], rgb_act), cg = act_rgb(v[1], rgb_act), cb = act_rgb(v[2], rgb_act);
 		const float weight = st.alpha[j] * T_before;
-		const float T = after.x;
+		const float T = T_before * (1.f - st.alpha[j]);          // the chain's own update (ray_marcher.cu:181)
 		const float d0 = A.K.loss_scale * ((weight * og.x) * act_rgb_derivative(v[0], rgb_act) + srf_max(0.0f, l2_reg * v[0]));
 		const float d1 = A.K.loss_scale * ((weight * og.y) * act_rgb_derivative(v[1], rgb_act) + srf_max(0.0f, l2_reg * v[1]));
 		const float d2 = A.K.loss_scale * ((weight * og.z) * act_rgb_derivative(v[2], rgb_act) + srf_max(0.0f, l2_reg * v[2]));
@@ -539,7 +566,7 @@ SRF_HD void phase_c(uint32_t tid, uint32_t win, const Args& A, const Window<G>& 
 		const float dotv = (og.x * (T * cr - sx) + og.y * (T * cg - sy)) + og.z * (T * cb - sz);
 		const float dmlp = dd * (st.dt[j] * dotv);
 		const float d3 = A.K.loss_scale * dmlp + (v[3] < 0 ? -l1_reg_density : 0.0f);
-		const size_t o = (size_t)srf_f2u(og.w) + k;
+		const size_t o = (size_t)(uint32_t)(srf_f2u(og.w) + srel);
 		// One vector store per sample when the records are 4 wide (the reference's padded_output_width).  The general
 		// case goes through volatile pointers only to keep the compiler from folding both cases into scalar stores.
 		if (HALF_OUT) {
@@ -584,10 +611,9 @@ SRF_HD void coords_copy_rows(uint32_t lane, uint32_t q0, const Args& A, const Wi
 		if (q < total) {
 			const uint32_t r = w.owner[q];
 			if (r < RAYS) {
-				const uint32_t k = q - pl.rbase[r];
-				if (k < rl.out[r].n_kept) {
+				if (q < rl.out[r].s_end) {
 					ok[u] = true;
-					o[u] = (size_t)rl.out[r].cbase + k;
+					o[u] = (size_t)(uint32_t)(rl.out[r].obase + q);
 					for (int c = 0; c < 7; ++c) cc[u][c] = src[7 * q + c];
 				}
 			}

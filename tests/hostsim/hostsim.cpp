@@ -114,7 +114,7 @@ static void run_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n
 				if (!backward) {
 					for (uint32_t t = 0; t < RAYS; ++t) if (ray0 + t < B.n_active) side[ray0 + t] = rl.rnf[t];
 				} else {
-					for (uint32_t t = 0; t < RAYS; ++t) commit_ray(t, ray0, ray0 + t < B.n_active ? side[ray0 + t] : 0u, B, rl);
+					for (uint32_t t = 0; t < RAYS; ++t) commit_ray(t, ray0, ray0 + t < B.n_active ? side[ray0 + t] : 0u, B, rl, pl);
 					for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
 					for (uint32_t win = 0; win < n_win; ++win) {
 						for (uint32_t t = 0; t < GW::THREADS; ++t) phase_a<GW, HI>(t, win, B, *ww, pl, st_w[t]);
@@ -157,14 +157,15 @@ static void run_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n
 			for (uint32_t t = 0; t < RAYS; ++t) rn_max = pl.rn[t] > rn_max ? pl.rn[t] : rn_max;
 			for (uint32_t t = 0; t < RAYS; ++t) n[t] = count_lane<GS>(t, rn_max, A, w, pl);
 			for (uint32_t t = 0; t < RAYS; ++t) n_max = n[t] > n_max ? n[t] : n_max;
-			for (uint32_t t = 0; t < RAYS; ++t) chain_counted<GS>(t, n[t], n_max, w, rl, pl, c[t]);
+			for (uint32_t t = 0; t < RAYS; ++t) chain_counted<GS, false>(t, n[t], n_max, w, rl, pl, c[t]);
+			for (uint32_t t = 0; t < RAYS; ++t) mark_owners<GS>(t, rn_max, w, pl);
 			for (uint32_t t = 0; t < RAYS; ++t) finish_ray(t, ray0, A, rl, c[t], tgt[t], lo, hi);
 		} else {
 			for (uint32_t t = 0; t < RAYS; ++t) n[t] = ray0 + t < A.n_active ? side[ray0 + t] : 0u;
 		}
 		uint32_t run = prefix;
 		for (uint32_t t = 0; t < RAYS; ++t) {
-			if (fast) commit_ray(t, ray0, run, A, rl, lo, hi);
+			if (fast) commit_ray(t, ray0, run, A, rl, pl, lo, hi);
 			else if (ray0 + t < A.n_active) side[ray0 + t] = run;
 			run += n[t];
 		}
