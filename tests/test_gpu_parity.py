@@ -162,6 +162,87 @@ def test_training_sampler(gpu, orc, config_id, scale, budget, monkeypatch):
         assert np.array_equal(coords.cpu().numpy(), want["coords"])
 
 
+SAMPLER_VARIANTS = {
+    "log_stepping": dict(sampling_type="Log"),
+    "original_stepping_cone": dict(sampling_type="Original", cone_angle_constant=1 / 256),
+    "original_stepping_fixed": dict(sampling_type="Original", cone_angle_constant=0.0, maximum_marching_steps=512),
+    "ngp_warp": dict(warping_type="NGP", aabb_scale=4, sampling_type="Original", cone_angle_constant=1 / 256, far_distance=8.0),
+    "mipnerf360_warp": dict(warping_type="MipNeRF360"),
+    "donerf_warp": dict(warping_type="DONeRF"),
+    "sigmoid_warp": dict(warping_type="Sigmoid"),
+    "sinusoidal_warp": dict(warping_type="SinusoidalProjection"),
+    "reciprocal_grid": dict(grid_distribution_type="WarpedSpace_Reciprocal"),
+    "metric_exp_grid": dict(grid_distribution_type="MetricSpace_Exp"),
+    "metric_reciprocal_grid": dict(grid_distribution_type="MetricSpace_Reciprocal"),
+    "no_pixel_snap": dict(snap_to_pixel_centers_in_training=False, snap_to_pixel_centers_in_rendering=False),
+    "no_grid": dict(use_grid=False, maximum_marching_steps=64),
+}
+
+
+@pytest.mark.parametrize("variant", sorted(SAMPLER_VARIANTS))
+def test_sampler_settings_other_than_the_workloads(gpu, orc, variant):
+    """The stepping rules, warps, grid distributions and switches that none of the five workloads uses (occupancy_sampler.cu:302-326,
+    :381-436; common_device.h:380-411), on workload 2's bounded scene at a quarter of its size with a random bitfield: the training
+    march and one rendered frame against the oracle."""
+    torch = gpu
+    from sphericalrf_amd import api, scene
+    w = scene.workload(2, 0.25)
+    cfg = dict(w["sampler"], num_cascades=2, **SAMPLER_VARIANTS[variant])
+    p = helpers.oracle_params(orc, cfg)
+    rng = np.random.default_rng(sorted(SAMPLER_VARIANTS).index(variant))
+    s = api.OccupancySampler(cfg)
+    bf = None
+    if cfg.get("use_grid", True):
+        grid = (rng.random(p.n_total) < 0.15).astype(np.float32)
+        bf, _ = orc.update_grid_bitfield(p, grid)
+        s.set_density_grid(torch.from_numpy(grid).cuda())
+        s.update_grid_bitfield()
+        assert np.array_equal(s.density_grid_bitfield.cpu().numpy(), bf)
+    res = w["resolution"]
+    o_ds = orc.make_dataset(w["cameras"], res, w["focal"], (0.5, 0.5))
+    g_ds = api.Dataset(torch.from_numpy(w["cameras"]).cuda(), res, w["focal"], (0.5, 0.5))
+    n_rays, cap = 6000, 1 << 22
+    want = orc.generate_training_samples(p, n_rays, 3, cap, o_ds, bf, orc.pcg32(99), coords_capacity=cap)
+    rays, rgba = torch.zeros((n_rays, 6), device="cuda"), torch.zeros((n_rays, 4), device="cuda")
+    ns = torch.zeros((n_rays, 2), dtype=torch.int32, device="cuda")
+    coords = torch.zeros((cap, 7), device="cuda")
+    ts, dts, cell = torch.zeros(cap, device="cuda"), torch.zeros(cap, device="cuda"), torch.zeros(cap, dtype=torch.int32, device="cuda")
+    rc, nc = torch.zeros(1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    s.sample_coords_from_dataset(n_rays, 3, cap, g_ds, rays, rgba, rc, ns, coords, nc, api.Pcg32(99), ts, dts, cell)
+    torch.cuda.synchronize()
+    assert int(rc.item()) == want["ray_counter"] and int(u32(nc)[0]) == want["numsteps_counter"]
+    assert want["numsteps_counter"] > n_rays                                     # the variant really marches
+    assert np.array_equal(u32(ns), want["numsteps"])
+    assert np.array_equal(u32(cell), want["cell"])
+    assert np.array_equal(np.stack([ts.cpu().numpy(), dts.cpu().numpy()], axis=1), want["t_dt"])
+    assert np.array_equal(coords.cpu().numpy(), want["coords"])
+    cam = w["cameras"][0]
+    n = res[0] * res[1]
+    if variant.startswith("metric"):
+        # the stand-in field is addressed by warped position, which a metric-space grid does not pass on: first hits and one round of
+        # render coordinates instead (occupancy_sampler.cu:691-863)
+        pay = torch.zeros(n * 40, dtype=torch.uint8, device="cuda")
+        s.generate_rays_from_camera_matrix(res, w["focal"], (0.5, 0.5), cam, pay)
+        o_pay = orc.init_rays_with_payload(p, res, w["focal"], (0.5, 0.5), cam)
+        orc.advance_pos(p, o_pay, bf)
+        assert np.array_equal(pay.cpu().numpy().view(O.PAYLOAD_DTYPE), o_pay) and (o_pay["alive"] == 1).mean() > 0.2
+        g_coords, o_coords = torch.zeros((n * 4, 7), device="cuda"), np.zeros((n * 4, 7), np.float32)
+        s.generate_coords_from_rays(n, 4, pay, g_coords)
+        orc.generate_coords_from_rays(p, n, 4, bf, o_pay, o_coords)
+        assert np.array_equal(pay.cpu().numpy().view(O.PAYLOAD_DTYPE), o_pay) and np.array_equal(g_coords.cpu().numpy(), o_coords)
+        return
+    # one frame
+    table = scene.field_table(1024, 3)
+    table[:, 3] *= 10
+    want_frame, want_ns, _ = orc.render_frame(p, orc.make_field(table, 5), bf, res, w["focal"], (0.5, 0.5), cam, transmittance_threshold=1e-4, train_in_linear_colors=True)
+    m = api.RayMarcher(dict(train_in_linear_color=True, transmittance_threshold=1e-4))
+    frame = torch.ones((res[1], res[0], 4), device="cuda")
+    fns = torch.zeros(res[0] * res[1], dtype=torch.int32, device="cuda")
+    s.render_frame_fused(m, api.Field(torch.from_numpy(table).cuda(), 5), res, w["focal"], (0.5, 0.5), cam, frame, fns)
+    assert np.array_equal(u32(fns).reshape(res[1], res[0]), want_ns)
+    assert np.array_equal(frame.cpu().numpy(), want_frame)
+
+
 def test_full_size_march_is_the_same_with_and_without_the_empty_space_table(gpu, monkeypatch):
     """Workload 4's grid (512x256x256 x 5 cascades, 64 blocks per axis) and ray distribution: the march that skips
     probes through provably empty stretches and the one that probes every step give identical bytes."""
@@ -327,6 +408,45 @@ def test_loss_and_gradient(gpu, orc, hin, hout, variant):
     assert np.allclose(got.astype(np.float32), o_dloss.astype(np.float32), rtol=TOL, atol=1e-12)
     assert np.array_equal(got.view(np.uint16 if hout else np.uint32), o_dloss.view(np.uint16 if hout else np.uint32))
     assert np.array_equal(d_comp.cpu().numpy(), o_comp)
+
+
+@pytest.mark.parametrize("loss", ["L1", "Mape", "Smape", "SmoothL1", "LogL1", "RelativeL2"])
+@pytest.mark.parametrize("impl", ["stream", "unfused"])
+def test_every_loss_function(gpu, orc, loss, impl, monkeypatch):
+    """loss.cu:27-84: the six losses besides L2, through both compositing implementations, with sRGB targets, a visible background
+    and a capacity that clamps the last rays"""
+    torch = gpu
+    from sphericalrf_amd import api
+    from tests.test_fused_compositing_on_host import layout
+    monkeypatch.setenv("SRF_COMPOSITE_IMPL", impl)
+    o_loss_id = {"L1": O.LOSS_L1, "Mape": O.LOSS_MAPE, "Smape": O.LOSS_SMAPE, "SmoothL1": O.LOSS_SMOOTHL1, "LogL1": O.LOSS_LOGL1, "RelativeL2": O.LOSS_RELATIVEL2}[loss]
+    rng = np.random.default_rng(o_loss_id + 60)
+    n_rays = 64 * 300 + 11
+    counts, base, total = layout(rng, "gaps", n_rays)
+    net = helpers.random_network_output(rng, total, np.float16)
+    dt = (rng.random(total) * 0.3 + 0.01).astype(np.float32)
+    tgt = rng.random((n_rays, 4)).astype(np.float32)
+    cap = int(counts.sum() * 0.95)
+    a = loss_args(n_rays, cap, network_output_dtype=O.DTYPE_F16, loss_type=o_loss_id, color_space=O.COLOR_SRGB, train_in_linear_color=0,
+                  background_color=(O.f32 * 3)(0.3, 0.5, 0.7), rgb_activation=O.ACT_LOGISTIC, density_activation=O.ACT_EXPONENTIAL, mean_density=0.5)
+    idx = np.stack([counts, base], axis=1).astype(np.uint32)
+    o_idx, o_dloss = idx.copy(), np.zeros((cap, 4), np.float32)
+    o_lossv, o_rgb = np.full(n_rays, -1, np.float32), np.zeros((n_rays, 3), np.float32)
+    o_total = orc.volume_rendering_with_loss_and_gradient(a, tgt, n_rays, o_idx, dt, net, o_dloss, loss_output=o_lossv, rgb_ray_out=o_rgb)
+    m = api.RayMarcher(dict(train_with_random_bg_color=False, train_in_linear_color=False, transmittance_threshold=1e-4))
+    d_idx = torch.from_numpy(idx.view(np.int32)).cuda()
+    d_dloss = torch.zeros((cap, 4), device="cuda")
+    d_loss, d_rgb = torch.full((n_rays,), -1.0, device="cuda"), torch.zeros((n_rays, 3), device="cuda")
+    cnt = torch.zeros(1, dtype=torch.int32, device="cuda")
+    nrc = torch.full((1,), n_rays, dtype=torch.int32, device="cuda")
+    m.volume_rendering_with_loss_and_gradient(n_rays, cap, torch.from_numpy(tgt).cuda(), nrc, d_idx, torch.from_numpy(dt).cuda(), torch.from_numpy(net).cuda(), d_dloss, cnt,
+                                              rgb_activation=api.ACT_LOGISTIC, density_activation=api.ACT_EXPONENTIAL, loss_output=d_loss, loss_type=loss,
+                                              density_grid_mean=torch.full((1,), 0.5, device="cuda"), background_color=(0.3, 0.5, 0.7), color_space=api.COLOR_SRGB, rgb_ray_out=d_rgb)
+    m.sync_check()
+    assert int(cnt.item()) == o_total and np.array_equal(u32(d_idx), o_idx)
+    assert np.array_equal(d_rgb.cpu().numpy().view(np.uint32), o_rgb.view(np.uint32)) and np.array_equal(d_loss.cpu().numpy().view(np.uint32), o_lossv.view(np.uint32))
+    assert np.array_equal(d_dloss.cpu().numpy().view(np.uint32), o_dloss.view(np.uint32))
+    assert np.abs(o_dloss).max() > 0
 
 
 @pytest.mark.parametrize("config_id,scale", [(1, 0.5), (2, 0.25), (2, 1.0), (3, 0.125)])
