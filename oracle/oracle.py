@@ -283,6 +283,13 @@ class Oracle:
         self.lib.orc_generate_grid_samples(C.byref(p), u32(n_elements), rng, u32(step), _ptr(grid_in, np.float32, p.n_total), f32(thresh), _ptr(pos), _ptr(idx))
         return pos, idx
 
+    def mark_untrained_density_grid(self, p, resolution, focal_length, xforms):
+        xforms = np.ascontiguousarray(xforms, dtype=np.float32).reshape(-1, 12)
+        grid = np.empty(p.n_total, np.float32)
+        self.lib.orc_mark_untrained_density_grid(C.byref(p), u32(xforms.shape[0]), (i32 * 2)(*resolution), (f32 * 2)(*focal_length),
+                                                 _ptr(xforms, np.float32, allow_none=True), _ptr(grid))
+        return grid
+
     def splat_grid_samples(self, p, indices, padded_output_width, network_output, density_activation, grid_current):
         dtype = DTYPE_F16 if network_output.dtype == np.float16 else DTYPE_F32
         n = indices.size

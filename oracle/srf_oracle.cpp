@@ -791,6 +791,62 @@ void orc_generate_grid_samples(const orc_params* Pp, uint32_t n_elements, orc_pc
 	}
 }
 
+// internal/sampler/occupancy_sampler.cu:12-102 — mark_untrained_density_grid: 0 where some training camera sees the cell, -1 elsewhere.
+// The switch over the grid distribution is restated with its fall-through (:52-57: MetricSpace_Exp has no break and runs into
+// MetricSpace_Reciprocal's two statements as well).  The reference's grid is cubic; here the cell centre uses each axis' own size and
+// the voxel radius the first axis' (the same thing for a cubic grid).  xforms: n_images column-major 3x4 matrices.
+void orc_mark_untrained_density_grid(const orc_params* Pp, uint32_t n_images, const int32_t resolution[2], const float focal_length[2],
+                                     const float* xforms, float* grid_out) {
+	const orc_params& P = *Pp;
+	const uint32_t n_grid_elements = n_cells(P);
+	const uint32_t n_elements = n_grid_elements * P.n_cascades;
+	for (uint32_t i = 0; i < n_elements; ++i) {
+		const uint32_t level = i / n_grid_elements, pos_idx = i % n_grid_elements;
+		const uint32_t x = morton3d_invert(pos_idx >> 0), y = morton3d_invert(pos_idx >> 1), z = morton3d_invert(pos_idx >> 2);
+		V3 pos{((float)x + 0.5f) / (float)P.grid_size[0] - 0.5f, ((float)y + 0.5f) / (float)P.grid_size[1] - 0.5f, ((float)z + 0.5f) / (float)P.grid_size[2] - 0.5f};
+		const V3 half{0.5f, 0.5f, 0.5f};
+		switch (P.griddist_type) {
+		case ORC_GRID_WARPED_EXP:
+			pos = pos * srf_exp2i(-(int)(P.n_cascades - level - 1));
+			pos = pos + half;
+			pos = unwarp_position(P, pos);
+			break;
+		case ORC_GRID_WARPED_RECIPROCAL:
+			pos = V3{pos.x / (float)(P.n_cascades - level), pos.y / (float)(P.n_cascades - level), pos.z / (float)(P.n_cascades - level)};
+			pos = pos + half;
+			pos = unwarp_position(P, pos);
+			break;
+		case ORC_GRID_METRIC_EXP:
+			pos = pos * ((float)P.aabb_scale * srf_exp2i(-(int)(P.n_cascades - level - 1)));
+			pos = pos + half;
+			/* falls through, as in the reference */
+		case ORC_GRID_METRIC_RECIPROCAL:
+			pos = pos * ((float)P.aabb_scale / (float)(P.n_cascades - level));
+			pos = pos + half;
+		default: break;
+		}
+		const float half_resx = (float)resolution[0] * 0.5f, half_resy = (float)resolution[1] * 0.5f;
+		float voxel_radius = 0.5f * 1.73205080757f * (float)P.aabb_scale / (float)P.grid_size[0];
+		switch (P.griddist_type) {
+		case ORC_GRID_WARPED_EXP: case ORC_GRID_METRIC_EXP: voxel_radius *= srf_exp2i(-(int)(P.n_cascades - level - 1)); break;
+		case ORC_GRID_WARPED_RECIPROCAL: case ORC_GRID_METRIC_RECIPROCAL: voxel_radius /= (float)(P.n_cascades - level); break;
+		default: break;
+		}
+		int count = 0;
+		for (uint32_t j = 0; j < n_images; ++j) {
+			const float* m = xforms + 12 * (size_t)j;
+			const V3 ploc = pos - V3{m[9], m[10], m[11]};
+			const float cx = (ploc.x * m[0] + ploc.y * m[1]) + ploc.z * m[2];
+			const float cy = (ploc.x * m[3] + ploc.y * m[4]) + ploc.z * m[5];
+			const float cz = (ploc.x * m[6] + ploc.y * m[7]) + ploc.z * m[8];
+			if (cz > 0.f) {
+				if (fabsf(cx) - voxel_radius < cz / focal_length[0] * half_resx && fabsf(cy) - voxel_radius < cz / focal_length[1] * half_resy) { ++count; break; }
+			}
+		}
+		grid_out[i] = count > 0 ? 0.f : -1.f;
+	}
+}
+
 // internal/sampler/occupancy_sampler.cu:187-212 — splat (max of non-negative floats == max of bit patterns)
 void orc_splat_grid_samples(const orc_params* Pp, uint32_t n_elements, const uint32_t* indices, uint32_t padded_output_width,
                             const void* network_output, int dtype, int density_activation, float* grid_current) {

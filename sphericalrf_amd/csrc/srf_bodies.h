@@ -64,6 +64,36 @@ SRF_HD uint64_t pixel_index(const float xy[2], const int32_t res[2], uint32_t im
 	return (uint64_t)px + (uint64_t)py * (uint64_t)res[0] + (uint64_t)img * (uint64_t)res[0] * (uint64_t)res[1];
 }
 
+// occupancy_sampler.cu:28-80 — where cell i of the cascaded grid lies in metric space and how far its corners reach, as the
+// camera-visibility mask sees them.  The reference's switch over the grid distribution falls through from MetricSpace_Exp into
+// MetricSpace_Reciprocal (:52-57), so a MetricSpace_Exp grid is scaled and shifted twice; that is kept.  (The reference's grid is
+// cubic: the radius uses the first axis' size.)
+SRF_HD void mask_cell(uint32_t i, const Params& P, Vec3* centre, float* radius) {
+	const uint32_t level = i / P.n_cells, cell = i % P.n_cells;
+	Vec3 p = mk3(((float)morton3d_invert(cell >> 0) + 0.5f) / (float)P.grid_size[0] - 0.5f,
+	             ((float)morton3d_invert(cell >> 1) + 0.5f) / (float)P.grid_size[1] - 0.5f,
+	             ((float)morton3d_invert(cell >> 2) + 0.5f) / (float)P.grid_size[2] - 0.5f);
+	const float shrink = srf_exp2i(-(int)(P.n_cascades - level - 1)), parts = (float)(P.n_cascades - level);
+	float r = 0.5f * 1.73205080757f * (float)P.aabb_scale / (float)P.grid_size[0];
+	const bool metric = P.griddist_type == SRF_GRID_METRIC_EXP || P.griddist_type == SRF_GRID_METRIC_RECIPROCAL;
+	if (P.griddist_type == SRF_GRID_WARPED_EXP) p = mk3(p.x * shrink + 0.5f, p.y * shrink + 0.5f, p.z * shrink + 0.5f);
+	else if (P.griddist_type == SRF_GRID_WARPED_RECIPROCAL) p = mk3(p.x / parts + 0.5f, p.y / parts + 0.5f, p.z / parts + 0.5f);
+	if (P.griddist_type == SRF_GRID_METRIC_EXP) { const float k = (float)P.aabb_scale * shrink; p = mk3(p.x * k + 0.5f, p.y * k + 0.5f, p.z * k + 0.5f); }
+	if (metric) { const float k = (float)P.aabb_scale / parts; p = mk3(p.x * k + 0.5f, p.y * k + 0.5f, p.z * k + 0.5f); }
+	else p = unwarp_position(P, p);
+	if (P.griddist_type == SRF_GRID_WARPED_EXP || P.griddist_type == SRF_GRID_METRIC_EXP) r *= shrink; else r /= parts;
+	*centre = p; *radius = r;
+}
+
+// occupancy_sampler.cu:82-99 — does the camera with the column-major 3x4 matrix m see a ball of that radius round the point
+SRF_HD bool mask_camera_sees(const float* m, Vec3 p, float radius, float focal_x, float focal_y, float half_res_x, float half_res_y) {
+	const Vec3 l = mk3(p.x - m[9], p.y - m[10], p.z - m[11]);
+	const float cx = (l.x * m[0] + l.y * m[1]) + l.z * m[2];
+	const float cy = (l.x * m[3] + l.y * m[4]) + l.z * m[5];
+	const float cz = (l.x * m[6] + l.y * m[7]) + l.z * m[8];
+	return cz > 0.f && srf_abs(cx) - radius < cz / focal_x * half_res_x && srf_abs(cy) - radius < cz / focal_y * half_res_y;
+}
+
 // ------------------------------------------------------------------------------------
 // occupancy_sampler.cu:104-185 — one candidate point: pick a cascade, probe up to ten
 // hashed cells for one above the threshold, jitter a point inside it.

@@ -23,6 +23,27 @@ int fill_u32(void* p, size_t n_words, uint32_t v, hipStream_t stream) {
 	return SRF_OK;
 }
 
+// occupancy_sampler.cu:12-102 — mark_untrained_density_grid: one thread per cell; the cameras pass through LDS a batch at a time, and a
+// workgroup stops as soon as every one of its cells has been seen by some camera
+constexpr uint32_t MASK_CAMERAS_PER_BATCH = 128;
+__global__ void __launch_bounds__(256) k_mark_untrained(Params P, uint32_t n_total, uint32_t n_images, float focal_x, float focal_y, float half_res_x, float half_res_y,
+                                                        const float* __restrict__ xforms, float* __restrict__ grid_out) {
+	__shared__ float cams[MASK_CAMERAS_PER_BATCH * 12];
+	const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+	Vec3 centre = mk3(0.f, 0.f, 0.f);
+	float radius = 0.f;
+	bool seen = i >= n_total;      // threads past the end have nothing to look for
+	if (i < n_total) mask_cell(i, P, &centre, &radius);
+	for (uint32_t first = 0; first < n_images; first += MASK_CAMERAS_PER_BATCH) {
+		const uint32_t n = n_images - first < MASK_CAMERAS_PER_BATCH ? n_images - first : MASK_CAMERAS_PER_BATCH;
+		for (uint32_t k = threadIdx.x; k < n * 12u; k += 256u) cams[k] = xforms[(size_t)first * 12u + k];
+		__syncthreads();
+		for (uint32_t j = 0; j < n && !seen; ++j) seen = mask_camera_sees(&cams[j * 12u], centre, radius, focal_x, focal_y, half_res_x, half_res_y);
+		if (__syncthreads_and(seen ? 1 : 0)) break;
+	}
+	if (i < n_total) grid_out[i] = seen ? 0.f : -1.f;
+}
+
 __global__ void __launch_bounds__(256) k_generate_grid_samples(Params P, uint32_t n_elements, Pcg32 rng, uint32_t step,
                                                                 const float* __restrict__ grid_in, float thresh,
                                                                 float* __restrict__ positions, uint32_t* __restrict__ indices, const uint32_t* __restrict__ above,
@@ -480,15 +501,20 @@ int srf_sampler_set_runtime(srf_sampler_t* s, int32_t snap_train, int32_t snap_r
 int srf_sampler_init(srf_sampler_t* s, uint32_t n_images, const int32_t image_resolution[2], const float focal_length[2],
                      const float principal_point[2], const float* camera_matrices, srf_pcg32* rng_host, void* stream) {
 	SRF_REQUIRE(s && rng_host, "srf_sampler_init: NULL argument");
-	(void)n_images; (void)image_resolution; (void)focal_length; (void)principal_point; (void)camera_matrices;
-	if (s->P.use_grid && s->init_grid_with_mask && s->P.warping_type == SRF_WARP_NGP)
-		SRF_FAIL(SRF_ERR_UNSUPPORTED, "srf_sampler_init: the camera-visibility mask of the NGP warp (mark_untrained_density_grid) is not implemented; set init_grid_with_mask=0");
+	(void)principal_point;
+	// occupancy_sampler.cu:959: the mask is only made for the NGP warp, where cameras and grid share a metric frame
+	const bool mask = s->P.use_grid && s->init_grid_with_mask && s->P.warping_type == SRF_WARP_NGP;
+	SRF_REQUIRE(!mask || (image_resolution && focal_length && (camera_matrices || n_images == 0)), "srf_sampler_init: the camera-visibility mask needs the cameras");
 	s->i_step = 0;
 	Pcg32 caller; caller.state = rng_host->state; caller.inc = rng_host->inc;
 	const uint32_t seed = pcg_next_uint(caller);
 	rng_host->state = caller.state; rng_host->inc = caller.inc;
 	pcg_seed(s->rng, (uint64_t)seed, 1u);
-	if (s->P.use_grid) {
+	if (mask) {
+		hipLaunchKernelGGL(k_mark_untrained, dim3(div_up(s->n_total, 256)), dim3(256), 0, (hipStream_t)stream, s->P, s->n_total, n_images, focal_length[0], focal_length[1],
+		                   (float)image_resolution[0] * 0.5f, (float)image_resolution[1] * 0.5f, camera_matrices, s->density_grid);
+		SRF_LAUNCH_CHECK();
+	} else if (s->P.use_grid) {
 		int rc = fill_u32(s->density_grid, s->n_total, 0u, (hipStream_t)stream);
 		if (rc != SRF_OK) return rc;
 	}

@@ -147,3 +147,90 @@ def test_grid_samples_fall_inside_their_cells(orc):
     pos2, idx2 = orc.generate_grid_samples(p, n, r, 3, grid, 2.0)
     want10 = ((i + 3 * n) * 56924617 + 9 * 19349663 + 96925573) % (1 << 32) % p.n_cells
     assert int(idx2[i]) % p.n_cells == want10
+
+
+# ---- camera-visibility mask (occupancy_sampler.cu:12-102) -----------------------------------------
+def _look_at(eye, target, up=(0.0, 0.0, 1.0)):
+    """column-major 3x4 camera-to-world matrix: columns are the camera's x, y, z axes (z = viewing direction) and its position"""
+    eye, target = np.asarray(eye, np.float64), np.asarray(target, np.float64)
+    z = target - eye
+    z /= np.linalg.norm(z)
+    x = np.cross(z, np.asarray(up, np.float64))
+    x /= np.linalg.norm(x)
+    y = np.cross(z, x)
+    return np.concatenate([x, y, z, eye]).astype(np.float32)
+
+
+def _mask_cell_centres(orc, p, griddist, aabb_scale):
+    """float64 centres and radii of all cells as the mask places them; MetricSpace_Exp is scaled and shifted twice, because the
+    reference's switch falls through into the MetricSpace_Reciprocal case (occupancy_sampler.cu:52-57)"""
+    N, C = np.array(p.grid_size[:3], np.float64), p.n_cascades
+    centres, radii = np.empty((p.n_total, 3)), np.empty(p.n_total)
+    for i in range(p.n_total):
+        level, cell = divmod(i, p.n_cells)
+        xyz = np.array([orc.morton3d_invert(cell), orc.morton3d_invert(cell >> 1), orc.morton3d_invert(cell >> 2)], np.float64)
+        q = (xyz + 0.5) / N - 0.5
+        shrink, parts = 2.0 ** (-(C - level - 1)), float(C - level)
+        r = 0.5 * np.sqrt(3.0) * aabb_scale / N[0]
+        if griddist == O.GRID_WARPED_EXP:
+            w = q * shrink + 0.5
+            q = (0.5 - 0.5 * aabb_scale) + w * aabb_scale            # the NGP warp is the affine map of the box onto the unit cube
+        elif griddist == O.GRID_WARPED_RECIPROCAL:
+            w = q / parts + 0.5
+            q = (0.5 - 0.5 * aabb_scale) + w * aabb_scale
+        elif griddist == O.GRID_METRIC_EXP:
+            q = (q * aabb_scale * shrink + 0.5) * (aabb_scale / parts) + 0.5
+        else:
+            q = q * (aabb_scale / parts) + 0.5
+        centres[i] = q
+        radii[i] = r * shrink if griddist in (O.GRID_WARPED_EXP, O.GRID_METRIC_EXP) else r / parts
+    return centres, radii
+
+
+@pytest.mark.parametrize("griddist", [O.GRID_WARPED_EXP, O.GRID_WARPED_RECIPROCAL, O.GRID_METRIC_EXP, O.GRID_METRIC_RECIPROCAL])
+def test_camera_visibility_mask_against_plane_distances(orc, griddist):
+    """A cell is kept (0) when, for some camera, it lies in front of the camera and its centre is closer than the cell's radius,
+    measured along the image axis, to the inside of both pairs of side planes of the viewing pyramid.  Stated here through the signed
+    distances to those four planes in float64 (the planes through the camera with normals (+-1, 0, -k) and (0, +-1, -k),
+    k = half the image size over the focal length); cells within 1e-4 of the decision are not judged."""
+    aabb_scale = 4
+    p = orc.params(aabb_scale=aabb_scale, grid_size=(8, 8, 8), n_cascades=2, warping_type=O.WARP_NGP, griddist_type=griddist,
+                   sampling_type=O.SAMPLING_ORIGINAL, n_max_steps=64)
+    res, focal = (64, 48), (150.0, 190.0)
+    rng = np.random.default_rng(griddist + 10)
+    cams = np.stack([_look_at(rng.uniform(-3, 4, 3), rng.uniform(-1, 2, 3)) for _ in range(3)])
+    got = orc.mark_untrained_density_grid(p, res, focal, cams)
+    assert set(np.unique(got)) <= {0.0, -1.0}
+    centres, radii = _mask_cell_centres(orc, p, griddist, aabb_scale)
+    seen = np.zeros(p.n_total, bool)
+    unsure = np.zeros(p.n_total, bool)
+    for m in cams.astype(np.float64):
+        ax, ay, az, eye = m[0:3], m[3:6], m[6:9], m[9:12]
+        local = centres - eye
+        X, Y, Z = local @ ax, local @ ay, local @ az
+        margins = [Z]
+        for coord, k in ((X, res[0] * 0.5 / focal[0]), (Y, res[1] * 0.5 / focal[1])):
+            norm = np.sqrt(1 + k * k)
+            outside = np.maximum(coord - k * Z, -coord - k * Z) / norm       # signed distance to the nearer side plane, positive outside
+            margins.append(radii / norm - outside)
+        margin = np.minimum.reduce(margins)
+        seen |= margin > 0
+        unsure |= np.abs(margin) < 1e-4
+    ok = ~unsure
+    assert np.array_equal(got[ok] == 0.0, seen[ok])
+    assert 0.02 < seen.mean() < 0.98 and ok.mean() > 0.98
+
+
+def test_camera_visibility_mask_special_cases(orc):
+    p = orc.params(aabb_scale=2, grid_size=(8, 8, 8), n_cascades=1, warping_type=O.WARP_NGP, griddist_type=O.GRID_WARPED_EXP,
+                   sampling_type=O.SAMPLING_ORIGINAL, n_max_steps=64)
+    centre = np.array([0.5, 0.5, 0.5])
+    # no camera sees nothing
+    assert (orc.mark_untrained_density_grid(p, (32, 32), (20.0, 20.0), np.zeros((0, 12), np.float32)) == -1.0).all()
+    # a distant camera with a wide view that looks at the box sees every cell; turned round it sees none
+    eye = centre + np.array([30.0, 0.0, 0.0])
+    assert (orc.mark_untrained_density_grid(p, (32, 32), (8.0, 8.0), _look_at(eye, centre)[None]) == 0.0).all()
+    assert (orc.mark_untrained_density_grid(p, (32, 32), (8.0, 8.0), _look_at(eye, 2 * eye - centre)[None]) == -1.0).all()
+    # one camera that sees is enough, wherever it stands in the list
+    cams = np.stack([_look_at(eye, 2 * eye - centre), _look_at(eye, centre)])
+    assert (orc.mark_untrained_density_grid(p, (32, 32), (8.0, 8.0), cams) == 0.0).all()
