@@ -288,6 +288,45 @@ int  srf_render_frame_fused(srf_sampler_t* s, const srf_marcher_t* m, const srf_
 int  srf_field_eval(const srf_sampler_t* s, const srf_field* field, uint32_t n_coords, const float* coords,
                     void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream);
 
+/* ---------------- a whole frame, library side ---------------- */
+/* What a caller's network does between srf_sampler_generate_coords_from_rays and srf_marcher_volume_rendering
+ * (m_network->inference_mixed_precision, internal/testbed.cu:552-556): n_elements coordinates of 7 floats in, one row of
+ * padded_output_width values of `dtype` per coordinate out, enqueued on `stream`.  Returns 0, or a negative SRF_ERR_* code
+ * (any other value is reported as SRF_ERR_INVALID). */
+typedef int (*srf_inference_fn)(void* user, uint32_t n_elements, const float* coords, void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream);
+
+typedef struct srf_frame_args {
+	int32_t  resolution[2];
+	float    focal_length[2], principal_point[2];
+	float    camera_matrix[12];          /* column-major 3x4, host memory */
+	uint32_t spp;
+	int32_t  render_mode, density_activation, rgb_activation;
+	float    depth_scale;                /* 1 / scene_scale (testbed.cu:577) */
+	int32_t  network_output_dtype;
+	uint32_t padded_output_width;
+} srf_frame_args;
+
+/* Testbed::render_frame up to and including shade_kernel, internal/testbed.cu:479-611: rays from the camera, then rounds of
+ * compact_rays / generate_coords_from_rays / inference / volume_rendering with n_steps = clamp(n_pixels / n_alive, 1, 8) until no ray
+ * is alive, then shade into frame_buffer (4 floats a pixel, cleared first).  The marcher owns the ray, coordinate and network-output
+ * buffers.  Like the reference it waits for the stream once a round to read the number of rays left.  *n_iterations (may be NULL)
+ * receives the number of rounds. */
+int  srf_render_frame(srf_sampler_t* s, srf_marcher_t* m, const srf_frame_args* args, srf_inference_fn inference, void* user,
+                      float* frame_buffer, uint32_t* n_iterations, void* stream);
+
+/* an srf_inference_fn that evaluates the stand-in field (srf_field_eval); user points at an srf_field_inference_ctx */
+typedef struct srf_field_inference_ctx { const srf_sampler_t* sampler; const srf_field* field; } srf_field_inference_ctx;
+int  srf_field_inference(void* user, uint32_t n_elements, const float* coords, void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream);
+
+/* CudaRenderBuffer::accumulate, internal/utils/render_buffer.cu:46-85, :211-227: running mean of the frames of one view.  spp is the
+ * number of frames already accumulated (0: the buffer is cleared first); the caller counts. */
+enum { SRF_TONEMAP_IDENTITY = 0, SRF_TONEMAP_ACES = 1, SRF_TONEMAP_HABLE = 2, SRF_TONEMAP_REINHARD = 3 };
+int  srf_frame_accumulate(const int32_t resolution[2], const float* frame_buffer, float* accumulate_buffer, uint32_t spp, int32_t color_space, void* stream);
+/* CudaRenderBuffer::tonemap, internal/utils/render_buffer.cu:87-178, :229-235: exposure, background (sRGB, premultiplied by its alpha
+ * through the remaining transparency), tone curve, output encoding.  out_rgba takes the place of the reference's CUDA surface. */
+int  srf_frame_tonemap(const int32_t resolution[2], float exposure, const float background_color[4], const float* accumulate_buffer,
+                       int32_t color_space, int32_t output_color_space, int32_t tonemap_curve, float* out_rgba, void* stream);
+
 /* ---------------- test hooks ---------------- */
 /* number of polls a workgroup of the streaming compositing kernel makes before it gives up waiting for its predecessors
  * (default 2^22).  0 lets a test exercise the give-up path without any kernel waiting for long. */

@@ -174,4 +174,20 @@ inline void shade(uint32_t n_rays, const float* rgba, const srf_ray_payload* pay
 	check(srf_shade(n_rays, rgba, payloads, frame_buffer, render_mode, train_in_linear_colors ? 1 : 0, stream));
 }
 
+// Testbed::render_frame up to shade (internal/testbed.cu:479-611); returns the number of rounds
+inline uint32_t render_frame(const OccupancySampler& sampler, const RayMarcher& marcher, const srf_frame_args& args, srf_inference_fn inference, void* user,
+                             float* frame_buffer, void* stream) {
+	uint32_t rounds = 0;
+	check(srf_render_frame(sampler.handle(), marcher.handle(), &args, inference, user, frame_buffer, &rounds, stream));
+	return rounds;
+}
+// CudaRenderBuffer::accumulate / ::tonemap (internal/utils/render_buffer.cu:46-235)
+inline void frame_accumulate(const int32_t resolution[2], const float* frame_buffer, float* accumulate_buffer, uint32_t spp, int32_t color_space, void* stream) {
+	check(srf_frame_accumulate(resolution, frame_buffer, accumulate_buffer, spp, color_space, stream));
+}
+inline void frame_tonemap(const int32_t resolution[2], float exposure, const float background_color[4], const float* accumulate_buffer, int32_t color_space,
+                          int32_t output_color_space, int32_t tonemap_curve, float* out_rgba, void* stream) {
+	check(srf_frame_tonemap(resolution, exposure, background_color, accumulate_buffer, color_space, output_color_space, tonemap_curve, out_rgba, stream));
+}
+
 } // namespace srf

@@ -417,6 +417,16 @@ class Oracle:
         self.lib.orc_field_eval(C.byref(p), C.byref(field), _f3(wpos), out)
         return np.array(out[:], dtype=np.float32)
 
+    def accumulate(self, frame, acc, sample_count, color_space):
+        """render_buffer.cu:46-85 in place on `acc` (float32 [n, 4])"""
+        self.lib.orc_accumulate(u32(frame.shape[0]), _ptr(frame, np.float32), _ptr(acc, np.float32), f32(sample_count), int(color_space))
+
+    def tonemap(self, acc, exposure, background_color, color_space, output_color_space, curve):
+        out = np.empty_like(acc)
+        self.lib.orc_tonemap(u32(acc.shape[0]), f32(exposure), (f32 * 4)(*background_color), _ptr(acc, np.float32), int(color_space), int(output_color_space),
+                             int(curve), _ptr(out))
+        return out
+
     def render_frame(self, p, field, bitfield, res, focal, pp, cam, spp=0, transmittance_threshold=1e-4, train_in_linear_colors=True):
         n = res[0] * res[1]
         frame = np.zeros((res[1], res[0], 4), np.float32)

@@ -1391,6 +1391,80 @@ void orc_shade(uint32_t n, const float* rgba, const orc_payload* payloads, float
 	}
 }
 
+// internal/utils/render_buffer.cu:46-85 — accumulate_kernel over all pixels (SRGB falls through into Linear on purpose)
+void orc_accumulate(uint32_t n_pixels, const float* frame_buffer, float* accumulate_buffer, float sample_count, int color_space) {
+	for (uint32_t i = 0; i < n_pixels; ++i) {
+		float color[4], tmp[4];
+		for (int c = 0; c < 4; ++c) { color[c] = frame_buffer[4 * (size_t)i + c]; tmp[c] = accumulate_buffer[4 * (size_t)i + c]; }
+		switch (color_space) {
+		case ORC_COLOR_VISPOSNEG: {
+			float val = color[0] - color[1];
+			float tmp_val = tmp[0] - tmp[1];
+			tmp_val = (tmp_val * sample_count + val) / (sample_count + 1);
+			tmp[0] = fmaxf(tmp_val, 0.0f);
+			tmp[1] = fmaxf(-tmp_val, 0.0f);
+		} break;
+		case ORC_COLOR_SRGB:
+			for (int c = 0; c < 3; ++c) color[c] = linear_to_srgb(color[c]);
+			/* fall through */
+		case ORC_COLOR_LINEAR:
+			for (int c = 0; c < 3; ++c) tmp[c] = (tmp[c] * sample_count + color[c]) / (sample_count + 1);
+			break;
+		}
+		tmp[3] = (tmp[3] * sample_count + color[3]) / (sample_count + 1);
+		for (int c = 0; c < 4; ++c) accumulate_buffer[4 * (size_t)i + c] = tmp[c];
+	}
+}
+
+// internal/utils/render_buffer.cu:87-140 — tonemap(): 0 Identity, 1 ACES, 2 Hable, 3 Reinhard
+static void tonemap3(float x[3], int curve) {
+	if (curve == 0) return;
+	for (int c = 0; c < 3; ++c) x[c] = fmaxf(x[c], 0.f);
+	float k0, k1, k2, k3, k4, k5;
+	if (curve == 1) {
+		k0 = 0.6f * 0.6f * 2.51f; k1 = 0.6f * 0.03f; k2 = 0.0f; k3 = 0.6f * 0.6f * 2.43f; k4 = 0.6f * 0.59f; k5 = 0.14f;
+	} else if (curve == 2) {
+		const float A = 0.15f, B = 0.50f, C = 0.10f, D = 0.20f, E = 0.02f, F = 0.30f;
+		k0 = A * F - A * E; k1 = C * B * F - B * E; k2 = 0.0f; k3 = A * F; k4 = B * F; k5 = D * F * F;
+		const float W = 11.2f;
+		const float nom = k0 * (W * W) + k1 * W + k2;
+		const float denom = k3 * (W * W) + k4 * W + k5;
+		const float whiteScale = denom / nom;
+		k0 = 4.0f * k0 * whiteScale; k1 = 2.0f * k1 * whiteScale; k2 = k2 * whiteScale; k3 = 4.0f * k3; k4 = 2.0f * k4;
+	} else {
+		float Y = (0.2126f * x[0] + 0.7152f * x[1]) + 0.0722f * x[2];
+		float inv = 1.f / (Y + 1.0f);
+		for (int c = 0; c < 3; ++c) x[c] = x[c] * inv;
+		return;
+	}
+	for (int c = 0; c < 3; ++c) {
+		float colSq = x[c] * x[c];
+		float nom = (colSq * k0 + k1 * x[c]) + k2;
+		float denom = (k3 * colSq + k4 * x[c]) + k5;
+		x[c] = nom / denom;
+	}
+}
+
+// internal/utils/render_buffer.cu:142-178 — tonemap_kernel over all pixels, writing floats where the reference writes a surface
+void orc_tonemap(uint32_t n_pixels, float exposure, const float background_color[4], const float* accumulate_buffer, int color_space,
+                 int output_color_space, int tonemap_curve, float* out) {
+	const float scale = e_pow(2.0f, exposure);
+	for (uint32_t i = 0; i < n_pixels; ++i) {
+		float color[4];
+		for (int c = 0; c < 4; ++c) color[c] = accumulate_buffer[4 * (size_t)i + c];
+		for (int c = 0; c < 3; ++c) color[c] *= scale;
+		float bg[4] = {background_color[0], background_color[1], background_color[2], background_color[3]};
+		if (color_space != ORC_COLOR_SRGB) for (int c = 0; c < 3; ++c) bg[c] = srgb_to_linear(bg[c]);
+		float weight = (1 - color[3]) * bg[3];
+		for (int c = 0; c < 3; ++c) color[c] += bg[c] * weight;
+		color[3] += weight;
+		if (color_space == ORC_COLOR_SRGB) for (int c = 0; c < 3; ++c) color[c] = srgb_to_linear(color[c]);
+		tonemap3(color, tonemap_curve);
+		if (output_color_space == ORC_COLOR_SRGB) for (int c = 0; c < 3; ++c) color[c] = linear_to_srgb(color[c]);
+		for (int c = 0; c < 4; ++c) out[4 * (size_t)i + c] = color[c];
+	}
+}
+
 // tiny-cuda-nn fill_rollover: elements past the valid prefix repeat it cyclically
 void orc_fill_rollover(uint32_t n_out, uint32_t width_bytes, uint32_t n_in, uint8_t* buf) {
 	if (n_in == 0) return;

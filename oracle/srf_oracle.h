@@ -120,6 +120,9 @@ void  orc_loss_and_gradient(int loss_type, const float target[3], const float pr
 /* ---- grid maintenance ---- */
 void  orc_generate_grid_samples(const orc_params* p, uint32_t n_elements, orc_pcg32 rng, uint32_t step,
                                 const float* grid_in, float thresh, float* positions_out, uint32_t* indices_out);
+void  orc_accumulate(uint32_t n_pixels, const float* frame_buffer, float* accumulate_buffer, float sample_count, int color_space);
+void  orc_tonemap(uint32_t n_pixels, float exposure, const float background_color[4], const float* accumulate_buffer, int color_space,
+                  int output_color_space, int tonemap_curve, float* out);
 void  orc_mark_untrained_density_grid(const orc_params* p, uint32_t n_images, const int32_t resolution[2], const float focal_length[2],
                                       const float* xforms, float* grid_out);
 void  orc_splat_grid_samples(const orc_params* p, uint32_t n_elements, const uint32_t* indices, uint32_t padded_output_width,

@@ -85,6 +85,22 @@ class Field(C.Structure):
     _fields_ = [("table", vp), ("table_size", u32), ("seed", u32)]
 
 
+class FrameArgs(C.Structure):
+    _fields_ = [
+        ("resolution", i32 * 2), ("focal_length", f32 * 2), ("principal_point", f32 * 2), ("camera_matrix", f32 * 12), ("spp", u32),
+        ("render_mode", i32), ("density_activation", i32), ("rgb_activation", i32), ("depth_scale", f32),
+        ("network_output_dtype", i32), ("padded_output_width", u32),
+    ]
+
+
+class FieldInferenceCtx(C.Structure):
+    _fields_ = [("sampler", vp), ("field", C.POINTER(Field))]
+
+
+# srf_inference_fn: (user, n_elements, coords, rgbsigma, dtype, padded_output_width, stream) -> int
+INFERENCE_FN = C.CFUNCTYPE(C.c_int, vp, u32, vp, vp, i32, u32, vp)
+
+
 # every symbol include/srf_hip.h declares
 SYMBOLS = [
     "srf_last_error", "srf_device_count",
@@ -95,6 +111,7 @@ SYMBOLS = [
     "srf_marcher_config_default", "srf_marcher_create", "srf_marcher_destroy", "srf_marcher_get_config", "srf_marcher_set_config",
     "srf_marcher_volume_rendering_with_loss_and_gradient", "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc", "srf_marcher_sync_check", "srf_marcher_volume_rendering",
     "srf_compact_rays", "srf_shade", "srf_fill_rollover", "srf_fill_rollover_and_rescale",
+    "srf_render_frame", "srf_field_inference", "srf_frame_accumulate", "srf_frame_tonemap",
     "srf_render_frame_fused", "srf_field_eval", "srf_debug_eval_elem", "srf_marcher_debug_set_lookback_spin_limit",
 ]
 
@@ -155,6 +172,10 @@ def load():
     L.srf_fill_rollover_and_rescale.argtypes = [u32, u32, vp, vp, i32, vp]
     L.srf_render_frame_fused.argtypes = [vp, vp, P(Field), P(i32 * 2), P(f32 * 2), P(f32 * 2), P(f32 * 12), u32, vp, vp, vp]
     L.srf_field_eval.argtypes = [vp, P(Field), u32, vp, vp, i32, u32, vp]
+    L.srf_render_frame.argtypes = [vp, vp, P(FrameArgs), vp, vp, vp, P(u32), vp]
+    L.srf_field_inference.argtypes = [vp, u32, vp, vp, i32, u32, vp]
+    L.srf_frame_accumulate.argtypes = [P(i32 * 2), vp, vp, u32, i32, vp]
+    L.srf_frame_tonemap.argtypes = [P(i32 * 2), f32, P(f32 * 4), vp, i32, i32, i32, vp, vp]
     L.srf_debug_eval_elem.argtypes = [i32, u32, vp, vp, vp, vp]
     for name in SYMBOLS:
         fn = getattr(L, name)

@@ -307,6 +307,50 @@ class OccupancySampler:
             _dev(frame_buffer, torch.float32, 4 * n, "frame_buffer"), _dev(n_samples, torch.int32, n, "n_samples", allow_none=True), _stream()))
 
 
+    def render_frame(self, marcher, inference, resolution, focal_length, principal_point, camera_matrix, frame_buffer, spp=0,
+                     render_mode=K.RENDER_SHADE, density_activation=K.ACT_EXPONENTIAL, rgb_activation=K.ACT_LOGISTIC, depth_scale=1.0,
+                     network_output_dtype=K.DTYPE_F16, padded_output_width=4):
+        """Testbed::render_frame up to shade (internal/testbed.cu:479-611).  `inference` is a Field (the stand-in network) or a callable
+        (n_elements, coords_ptr, rgbsigma_ptr, dtype, padded_output_width, stream_ptr) -> int that enqueues the network on the stream.
+        Returns the number of rounds."""
+        a = K.FrameArgs()
+        a.resolution, a.focal_length, a.principal_point = (K.i32 * 2)(*resolution), (K.f32 * 2)(*focal_length), (K.f32 * 2)(*principal_point)
+        a.camera_matrix = (K.f32 * 12)(*[float(v) for v in camera_matrix])
+        a.spp, a.render_mode, a.density_activation, a.rgb_activation = int(spp), int(render_mode), int(density_activation), int(rgb_activation)
+        a.depth_scale, a.network_output_dtype, a.padded_output_width = float(depth_scale), int(network_output_dtype), int(padded_output_width)
+        iters = K.u32(0)
+        n = resolution[0] * resolution[1]
+        if isinstance(inference, Field):
+            f = inference.as_c()
+            ctx = K.FieldInferenceCtx(self._h, C.pointer(f))
+            fn, user, keep = C.cast(self._L.srf_field_inference, C.c_void_p), C.cast(C.pointer(ctx), C.c_void_p), (f, ctx)
+        else:
+            cb = K.INFERENCE_FN(lambda user, n_el, coords, out, dtype, width, stream: int(inference(n_el, coords, out, dtype, width, stream) or 0))
+            fn, user, keep = C.cast(cb, C.c_void_p), None, (cb,)
+        K.check(self._L.srf_render_frame(self._h, marcher._h, C.byref(a), fn, user, _dev(frame_buffer, torch.float32, 4 * n, "frame_buffer"), C.byref(iters), _stream()))
+        del keep
+        return int(iters.value)
+
+
+def frame_accumulate(resolution, frame_buffer, accumulate_buffer, spp, color_space=K.COLOR_LINEAR):
+    """CudaRenderBuffer::accumulate (internal/utils/render_buffer.cu:46-85, :211-227); spp = frames already accumulated"""
+    n = resolution[0] * resolution[1]
+    K.check(K.load().srf_frame_accumulate(C.byref((K.i32 * 2)(*resolution)), _dev(frame_buffer, torch.float32, 4 * n, "frame_buffer"),
+                                          _dev(accumulate_buffer, torch.float32, 4 * n, "accumulate_buffer"), int(spp), int(color_space), _stream()))
+
+
+TONEMAP_IDENTITY, TONEMAP_ACES, TONEMAP_HABLE, TONEMAP_REINHARD = 0, 1, 2, 3
+
+
+def frame_tonemap(resolution, exposure, background_color, accumulate_buffer, out_rgba, color_space=K.COLOR_LINEAR, output_color_space=K.COLOR_SRGB,
+                  tonemap_curve=TONEMAP_IDENTITY):
+    """CudaRenderBuffer::tonemap (internal/utils/render_buffer.cu:87-178, :229-235)"""
+    n = resolution[0] * resolution[1]
+    K.check(K.load().srf_frame_tonemap(C.byref((K.i32 * 2)(*resolution)), float(exposure), C.byref((K.f32 * 4)(*background_color)),
+                                       _dev(accumulate_buffer, torch.float32, 4 * n, "accumulate_buffer"), int(color_space), int(output_color_space),
+                                       int(tonemap_curve), _dev(out_rgba, torch.float32, 4 * n, "out_rgba"), _stream()))
+
+
 class Field:
     """Table-lookup stand-in for the network (not in the reference): table is (size, 4) float32 on the GPU, size a power of two."""
 

@@ -8,7 +8,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIBDIR = os.path.join(_HERE, "lib")
 LIB = os.path.join(LIBDIR, "libsrf_hip.so")
-SOURCES = ["srf_common.hip", "srf_grid.hip", "srf_march.hip", "srf_composite.hip"]
+SOURCES = ["srf_common.hip", "srf_grid.hip", "srf_march.hip", "srf_composite.hip", "srf_frame.hip"]
 
 # -ffp-contract=off: a*b+c stays two rounded operations so host and device agree bit for bit.
 # packed-fp32-ops is switched off because some packed forms have produced wrong results on this hardware.

@@ -64,6 +64,67 @@ SRF_HD uint64_t pixel_index(const float xy[2], const int32_t res[2], uint32_t im
 	return (uint64_t)px + (uint64_t)py * (uint64_t)res[0] + (uint64_t)img * (uint64_t)res[0] * (uint64_t)res[1];
 }
 
+// ---- display post-process (internal/utils/render_buffer.cu) ----------------------------------
+// render_buffer.cu:46-85 — the running mean over the frames accumulated so far; an sRGB buffer takes the frame encoded
+SRF_HD Float4 accumulate_body(Float4 color, Float4 tmp, float sample_count, int32_t color_space) {
+	if (color_space == SRF_COLOR_VISPOSNEG) {
+		const float val = color.x - color.y;
+		float tmp_val = tmp.x - tmp.y;
+		tmp_val = (tmp_val * sample_count + val) / (sample_count + 1);
+		tmp.x = srf_max(tmp_val, 0.0f);
+		tmp.y = srf_max(-tmp_val, 0.0f);
+	} else {
+		if (color_space == SRF_COLOR_SRGB) { color.x = linear_to_srgb(color.x); color.y = linear_to_srgb(color.y); color.z = linear_to_srgb(color.z); }
+		tmp.x = (tmp.x * sample_count + color.x) / (sample_count + 1);
+		tmp.y = (tmp.y * sample_count + color.y) / (sample_count + 1);
+		tmp.z = (tmp.z * sample_count + color.z) / (sample_count + 1);
+	}
+	tmp.w = (tmp.w * sample_count + color.w) / (sample_count + 1);
+	return tmp;
+}
+
+struct TonemapArgs { float scale; float background[4]; int32_t color_space, output_color_space, curve; };
+
+// render_buffer.cu:87-140 — the tone curves: rational polynomials with the exposure bias and white point folded into their coefficients
+SRF_HD void tonemap_curve(float x[3], int32_t curve) {
+	if (curve == SRF_TONEMAP_IDENTITY) return;
+	for (int c = 0; c < 3; ++c) x[c] = srf_max(x[c], 0.f);
+	float k0, k1, k2, k3, k4, k5;
+	if (curve == SRF_TONEMAP_ACES) {
+		k0 = 0.6f * 0.6f * 2.51f; k1 = 0.6f * 0.03f; k2 = 0.0f; k3 = 0.6f * 0.6f * 2.43f; k4 = 0.6f * 0.59f; k5 = 0.14f;
+	} else if (curve == SRF_TONEMAP_HABLE) {
+		const float A = 0.15f, B = 0.50f, C = 0.10f, D = 0.20f, E = 0.02f, F = 0.30f, W = 11.2f;
+		k0 = A * F - A * E; k1 = C * B * F - B * E; k2 = 0.0f; k3 = A * F; k4 = B * F; k5 = D * F * F;
+		const float nom = k0 * (W * W) + k1 * W + k2, denom = k3 * (W * W) + k4 * W + k5;
+		const float white_scale = denom / nom;
+		k0 = 4.0f * k0 * white_scale; k1 = 2.0f * k1 * white_scale; k2 = k2 * white_scale; k3 = 4.0f * k3; k4 = 2.0f * k4;
+	} else {   // Reinhard, on the luminance
+		const float Y = (0.2126f * x[0] + 0.7152f * x[1]) + 0.0722f * x[2];
+		const float k = 1.f / (Y + 1.0f);
+		for (int c = 0; c < 3; ++c) x[c] = x[c] * k;
+		return;
+	}
+	for (int c = 0; c < 3; ++c) {
+		const float sq = x[c] * x[c];
+		const float nom = (sq * k0 + k1 * x[c]) + k2, denom = (k3 * sq + k4 * x[c]) + k5;
+		x[c] = nom / denom;
+	}
+}
+
+// render_buffer.cu:142-178 — one pixel from the accumulation buffer to the display buffer
+SRF_HD Float4 tonemap_body(Float4 color, const TonemapArgs& A) {
+	float rgb[3] = {color.x * A.scale, color.y * A.scale, color.z * A.scale};
+	float bg[3] = {A.background[0], A.background[1], A.background[2]};
+	if (A.color_space != SRF_COLOR_SRGB) for (int c = 0; c < 3; ++c) bg[c] = srgb_to_linear(bg[c]);     // the background colour is given in sRGB
+	const float weight = (1 - color.w) * A.background[3];
+	for (int c = 0; c < 3; ++c) rgb[c] += bg[c] * weight;
+	const float alpha = color.w + weight;
+	if (A.color_space == SRF_COLOR_SRGB) for (int c = 0; c < 3; ++c) rgb[c] = srgb_to_linear(rgb[c]);
+	tonemap_curve(rgb, A.curve);
+	if (A.output_color_space == SRF_COLOR_SRGB) for (int c = 0; c < 3; ++c) rgb[c] = linear_to_srgb(rgb[c]);
+	return mk4(rgb[0], rgb[1], rgb[2], alpha);
+}
+
 // occupancy_sampler.cu:28-80 — where cell i of the cascaded grid lies in metric space and how far its corners reach, as the
 // camera-visibility mask sees them.  The reference's switch over the grid distribution falls through from MetricSpace_Exp into
 // MetricSpace_Reciprocal (:52-57), so a MetricSpace_Exp grid is scaled and shifted twice; that is kept.  (The reference's grid is

@@ -876,6 +876,8 @@ void srf_marcher_destroy(srf_marcher_t* m) {
 	m->ws2.release();
 	m->reg.release();
 	m->compact_ws.release();
+	m->frame_ws.release();
+	if (m->frame_counter_host) (void)hipHostFree(m->frame_counter_host);
 	if (m->host_error) (void)hipHostFree((void*)m->host_error);
 	delete m;
 }

@@ -69,6 +69,8 @@ struct srf_marcher {
 	srf::Workspace ws2;         // per-ray forward results of the three-launch compositing
 	srf::Workspace reg;         // reg_distortion_buffer (ray_marcher.h:79-80)
 	srf::Workspace compact_ws;  // flags and positions of srf_marcher_compact_rays
+	srf::Workspace frame_ws;    // ray buffers, coordinates and network output of srf_render_frame
+	uint32_t* frame_counter_host = nullptr;  // pinned word through which srf_render_frame reads the ray counters
 	bool force_unfused = false;             // SRF_COMPOSITE_IMPL=unfused at creation
 	bool degraded = false;                  // the chain has failed once: every later call uses the three-launch implementation
 	volatile uint32_t* host_error = nullptr; // host word the streaming kernel raises when its chain gives up (pinned, device-writable)

@@ -543,6 +543,64 @@ def test_render_loop_and_fused_frame(gpu, orc, config_id, scale):
     assert np.array_equal(fb.cpu().numpy(), want_frame)
 
 
+@pytest.mark.parametrize("config_id,scale,inference", [(1, 0.5, "field"), (3, 0.125, "field"), (1, 0.25, "callback")])
+def test_library_side_frame_loop(gpu, orc, config_id, scale, inference):
+    """srf_render_frame (internal/testbed.cu:479-611) with the stand-in field as the network, handed over as the library's own
+    inference function or as a caller's callback: frame and number of rounds against the oracle's loop"""
+    torch = gpu
+    from sphericalrf_amd import api, scene, _capi
+    w, p, grid, bf, mean = helpers.build_scene(orc, config_id, scale)
+    s = make_sampler(torch, api, w, grid)
+    m = api.RayMarcher(dict(train_in_linear_color=False, transmittance_threshold=1e-4))
+    res, f, cam = w["resolution"], w["focal"], w["cameras"][-1]
+    table = scene.field_table(4096, 5)
+    table[:, 3] *= 20
+    want_frame, _, iters = orc.render_frame(p, orc.make_field(table, 77), bf, res, f, (0.5, 0.5), cam, transmittance_threshold=1e-4, train_in_linear_colors=False)
+    field = api.Field(torch.from_numpy(table).cuda(), 77)
+    calls = []
+    if inference == "callback":
+        fc = field.as_c()
+
+        def net(n_elements, coords, out, dtype, width, stream):      # a caller's network: raw device pointers in, work enqueued on the stream
+            calls.append(n_elements)
+            return _capi.load().srf_field_eval(s._h, fc, n_elements, coords, out, dtype, width, stream)
+    else:
+        net = field
+    frame = torch.ones((res[1], res[0], 4), device="cuda")
+    for rep in range(2):        # the second frame reuses the marcher's buffers
+        got_iters = s.render_frame(m, net, res, f, (0.5, 0.5), cam, frame, density_activation=api.ACT_NONE, rgb_activation=api.ACT_NONE,
+                                   network_output_dtype=api.DTYPE_F32)
+        assert got_iters == iters and np.array_equal(frame.cpu().numpy(), want_frame)
+    assert inference != "callback" or len(calls) == 2 * iters
+    assert (want_frame[..., 3] > 0).mean() > 0.05
+
+
+@pytest.mark.parametrize("color_space", [0, 1, 2])
+def test_accumulate_and_tonemap(gpu, orc, color_space):
+    """CudaRenderBuffer::accumulate and ::tonemap (internal/utils/render_buffer.cu:46-178): four frames into the running mean, then every
+    tone curve and both output encodings, against the oracle"""
+    torch = gpu
+    from sphericalrf_amd import api
+    res = (37, 21)
+    n = res[0] * res[1]
+    rng = np.random.default_rng(color_space)
+    o_acc = np.full((n, 4), 3.0, np.float32)
+    g_acc = torch.full((n, 4), 3.0, device="cuda")
+    for k in range(4):
+        frame = (rng.random((n, 4)) * 1.5).astype(np.float32)
+        if k == 0:
+            o_acc[:] = 0          # CudaRenderBuffer::accumulate clears the buffer before a view's first frame (render_buffer.cu:214-216)
+        orc.accumulate(frame, o_acc, float(k), color_space)
+        api.frame_accumulate(res, torch.from_numpy(frame).cuda(), g_acc, k, color_space)
+        assert np.array_equal(g_acc.cpu().numpy().view(np.uint32), o_acc.view(np.uint32))
+    for curve in (api.TONEMAP_IDENTITY, api.TONEMAP_ACES, api.TONEMAP_HABLE, api.TONEMAP_REINHARD):
+        for out_space in (api.COLOR_LINEAR, api.COLOR_SRGB):
+            want = orc.tonemap(o_acc, 0.7, (0.2, 0.5, 0.8, 0.6), color_space, out_space, curve)
+            out = torch.zeros((n, 4), device="cuda")
+            api.frame_tonemap(res, 0.7, (0.2, 0.5, 0.8, 0.6), g_acc, out, color_space, out_space, curve)
+            assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
 def test_render_after_the_grid_has_been_updated(gpu, orc):
     """workload 5's sequence at an eighth of its size: positions drawn from the grid, densities splatted and decayed into it,
     bitfield rebuilt, and then a frame marched through that bitfield (about half of it occupied, where the blob scenes
