@@ -176,7 +176,7 @@ __device__ inline uint32_t chain_resolve(const ChainScratch& S, uint32_t i, uint
 		const uint32_t gflag = (uint32_t)(vg >> 32), pflag = (uint32_t)(vp >> 32);
 		if (__ballot(gflag == 3u) != 0ull) { failed = true; break; }
 		if (!have_within && __ballot(gflag == 0u) == 0ull) {
-			within = wave_sum_u32(lane < j ? (uint32_t)vg : 0u);
+			within = wave_sum_fast(lane < j ? (uint32_t)vg : 0u);
 			have_within = true;
 		}
 		if (!have_before) {
@@ -190,9 +190,9 @@ __device__ inline uint32_t chain_resolve(const ChainScratch& S, uint32_t i, uint
 			const uint32_t first_poisoned = poisoned ? (uint32_t)__builtin_ctzll(poisoned) : 64u;
 			if (first_poisoned < first_prefix && first_poisoned < first_missing) { failed = true; break; }
 			if (first_prefix < first_missing) {
-				before += wave_sum_u32(lane < first_prefix ? (uint32_t)vs : (lane == first_prefix ? (uint32_t)vp : 0u));
+				before += wave_sum_fast(lane < first_prefix ? (uint32_t)vs : (lane == first_prefix ? (uint32_t)vp : 0u));
 				have_before = true;
-			} else if (first_missing == 64u) { before += wave_sum_u32((uint32_t)vs); hi -= 64; continue; }   // 64 totals, no prefix yet: look further back
+			} else if (first_missing == 64u) { before += wave_sum_fast((uint32_t)vs); hi -= 64; continue; }   // 64 totals, no prefix yet: look further back
 		}
 		if (have_before && have_within) break;
 		if (++spins > S.spin_limit) { failed = true; break; }
@@ -236,14 +236,14 @@ __device__ __forceinline__ void plan_from_records(uint32_t lane, uint32_t g, U2 
 	const uint32_t ray0 = g * RAYS;
 	const uint32_t n_here = A.n_active > ray0 ? (A.n_active - ray0 < RAYS ? A.n_active - ray0 : RAYS) : 0;
 	const uint32_t rn = rec.x, rabs = rec.y;             // (0, 0) past the active count
-	const uint32_t s0 = n_here ? (uint32_t)__shfl((int)rabs, 0, WAVE) : 0u;
-	const uint32_t prev_rabs = (uint32_t)__shfl_up((int)rabs, 1, WAVE), prev_rn = (uint32_t)__shfl_up((int)rn, 1, WAVE);
+	const uint32_t s0 = n_here ? lane_value_u32(rabs, 0) : 0u;
+	const uint32_t prev_rabs = lane_below_u32(rabs), prev_rn = lane_below_u32(rn);
 	const uint64_t prev_end = lane ? (uint64_t)prev_rabs + prev_rn : (uint64_t)s0;
 	const bool mine = lane < n_here;
 	const bool out_of_order = mine && (uint64_t)rabs < prev_end;
-	const uint32_t sum = wave_sum_u32(mine ? rn : 0u);
+	const uint32_t sum = wave_sum_fast(mine ? rn : 0u);
 	const uint32_t last = n_here ? n_here - 1 : 0u;
-	const uint64_t end = n_here ? (uint64_t)(uint32_t)__shfl((int)rabs, (int)last, WAVE) + (uint32_t)__shfl((int)rn, (int)last, WAVE) : 0ull;
+	const uint64_t end = n_here ? (uint64_t)lane_value_u32(rabs, last) + lane_value_u32(rn, last) : 0ull;
 	const uint64_t total64 = end >= s0 ? end - s0 : 0ull;
 	const uint32_t total = total64 > 0xffffffffull ? 0xffffffffu : (uint32_t)total64;
 	const bool contiguous = __ballot(out_of_order) == 0ull && !((uint64_t)total > (uint64_t)sum + GAP_SLACK);
@@ -313,8 +313,8 @@ __global__ void __launch_bounds__(ITEMS_THREADS) k_chain_items(uint32_t n_rays_m
 	uint32_t before = 0;
 	for (uint32_t k = tid; k < g_first / PREPARE_WAVES; k += ITEMS_THREADS) before += S.prepare_sums[k];
 	const uint32_t n = word & 0xffu;
-	const uint32_t incl = wave_inclusive_scan_u32(n);
-	const uint32_t before_w = wave_sum_u32(before);
+	const uint32_t incl = wave_inclusive_scan_fast(n);
+	const uint32_t before_w = wave_sum_fast(before);
 	if (lane == WAVE - 1) { wave_total[wave] = incl; wave_before[wave] = before_w; }
 	__syncthreads();
 	uint32_t base = 0, all = 0;
@@ -575,20 +575,20 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 		if (ray_wave) {
 			if (has1) {
 				const uint32_t ray1 = pl1.misc[M_GROUP] * RAYS, lo1 = pl1.misc[M_LANE_LO], hi1 = pl1.misc[M_LANE_HI];
-				if (fast1) n_cur = count_lane<G>(lane, wave_max_u32(pl1.rn[lane]), A, w1, pl1);
+				if (fast1) n_cur = count_lane<G>(lane, wave_max_fast(pl1.rn[lane]), A, w1, pl1);
 				else n_cur = (ray1 + lane < A.n_active && lane >= lo1 && lane < hi1) ? S.side[ray1 + lane] : 0u;
-				incl_cur = wave_inclusive_scan_u32(n_cur);
-				total_cur = (uint32_t)__shfl((int)incl_cur, WAVE - 1, WAVE);
+				incl_cur = wave_inclusive_scan_fast(n_cur);
+				total_cur = lane_value_u32(incl_cur, WAVE - 1);
 				chain_publish(S, i_1, total_cur);
 				SRF_T(7);
-				if (fast1) chain_counted<G, false>(lane, n_cur, wave_max_u32(n_cur), w1, sh.rl, pl1, carry);
+				if (fast1) chain_counted<G, false>(lane, n_cur, wave_max_fast(n_cur), w1, sh.rl, pl1, carry);
 				peek = chain_peek(S, i_1);                            // needed in the next first half; the items before this one have published by now unless their workgroups lag
 				SRF_T(4);
 			}
 		} else if (plan_wave) {
 			// the plan first: it waits for records requested an iteration ago, and that wait must not include anything younger (see above)
 			plan_next(pl3);
-			if (fast1) mark_owners<G>(lane, wave_max_u32(pl1.rn[lane]), w1, pl1);     // which ray each sample of item it + 1 belongs to, for its phase C
+			if (fast1) mark_owners<G>(lane, wave_max_fast(pl1.rn[lane]), w1, pl1);     // which ray each sample of item it + 1 belongs to, for its phase C
 			SRF_T(4);
 			if (has1) {
 				const uint32_t ray1 = pl1.misc[M_GROUP] * RAYS;
