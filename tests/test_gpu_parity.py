@@ -725,7 +725,7 @@ def test_errors_are_reported_not_thrown_across_the_abi(gpu):
     with pytest.raises(api.SrfError, match="x >= y >= z"):
         api.OccupancySampler(dict(warping_type="ERP", grid_distribution_type="WarpedSpace_Exp", grid_size=(8, 16, 8)))
     s = api.OccupancySampler(dict(warping_type="NGP", grid_distribution_type="WarpedSpace_Exp", grid_size=8))
-    with pytest.raises(api.SrfError, match="mark_untrained_density_grid"):
+    with pytest.raises(api.SrfError, match="needs the cameras"):      # the visibility mask is on by default
         s.init(1, (4, 4), (1.0, 1.0), (0.5, 0.5), None, None, api.Pcg32(1))
 
 
