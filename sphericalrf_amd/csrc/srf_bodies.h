@@ -801,77 +801,152 @@ SRF_HD void init_ray_body(uint32_t x, uint32_t y, const Params& P, const PixelAr
 	}
 }
 
-// occupancy_sampler.cu:738-797 — jitter the start, then step to the first occupied cell
-// After a probe at t found an empty cell and the step to the next t has been taken: walks t through the further
-// steps the empty-space table proves empty (the reference would probe each, find nothing and add its dt,
-// occupancy_sampler.cu:762-790).  Returns false when the march ends on a zero step.
-SRF_HD bool march_through_empty(const Params& P, float& t, float t_limit, float cone) {
+// ------------------------------------------------------------------------------------
+// The march the three render kernels share, as a lane state machine like the counting march above.  A probe looks the
+// cell at t up and, for an empty one, asks the empty-space table how far nothing can be found; steps then walk t through
+// that stretch without lookups (the reference would probe each, find nothing and add its dt,
+// occupancy_sampler.cu:762-790, :820-850).  What an occupied cell means is the caller's: hit(L, s) says how the march
+// goes on.  A wavefront runs its lanes' phases by majority (srf_march.hip); one lane alone runs them in turn.
+// ------------------------------------------------------------------------------------
+enum MarchEnd : uint32_t { MARCH_GOES_ON = 0, MARCH_LEFT_BOX = 1, MARCH_ZERO_STEP = 2, MARCH_STOPPED = 3, MARCH_NO_RAY = 4 };
+struct MarchLane { uint32_t phase; Vec3 o, d; float t, t_limit; SkipRay sr; };
+
+SRF_HD void march_start(MarchLane& L, Vec3 o, Vec3 d, float t, bool skipping) {
+	L.o = o; L.d = d;
+	L.t = L.t_limit = t;
+	if (skipping) L.sr = skip_ray_setup(o, d);
+	L.phase = LANE_PROBE;
+}
+
+template <class Hit>
+SRF_HD MarchEnd march_probe(MarchLane& L, const Params& P, const uint8_t* bitfield, const SkipTable& skip, bool skipping, const Hit& hit) {
+	const float cone = P.cone_angle_constant;
+	const Vec3 pos = along(L.o, L.d, L.t);
+	if (!aabb_contains(P, pos)) return MARCH_LEFT_BOX;
+	const Probe s = probe_at(P, bitfield, pos, L.t, cone, &skip);
+	L.t_limit = L.t;      // steps at t' < t_limit are known to find an empty cell
+	if (s.occ) return hit(L, s);
+	if (skipping) L.t_limit = skip_limit(P, skip, L.sr, L.o, L.d, L.t, s.radius, s.level);
+	L.t += s.dt;
+	if (s.dt == 0.f) return MARCH_ZERO_STEP;
+	L.phase = L.t < L.t_limit ? LANE_STEP : LANE_PROBE;
+	return MARCH_GOES_ON;
+}
+
+// the steps below t_limit, each lane for itself; the step sizes are count_steps's (the short form of the disparity chain
+// where it holds, calc_dt elsewhere), and a step of size zero ends the march.  The plain loop that lanes leave one by one
+// (seven vector instructions a step) beats predicated bursts of a fixed length here, where all lanes step before any probes.
+SRF_HD MarchEnd march_steps(MarchLane& L, const Params& P) {
+	const float cone = P.cone_angle_constant;
 	const ShortForm f = disparity_short_form(P);
-	if (f.usable && t >= f.t_lo) {
-		// the steps that start inside the short form's range, where steps are positive; what lies beyond goes step by step
-		const float lim = srf_min(t_limit, f.t_hi);
-		ShortChain ch = short_chain_at(t);
+	if (f.usable && L.t >= f.t_lo) {
+		const float lim = srf_min(L.t_limit, f.t_hi);
+		ShortChain ch = short_chain_at(L.t);
 		while (ch.t < lim) ch = short_chain_next(f, ch);
-		t = ch.t;
+		L.t = ch.t;
 	}
-	while (t < t_limit) {
-		const float dt = calc_dt(P, t, cone);
-		t += dt;
-		if (dt == 0.f) return false;
+	while (L.t < L.t_limit) {      // what the short form does not cover
+		const float dt = calc_dt(P, L.t, cone);
+		L.t += dt;
+		if (dt == 0.f) return MARCH_ZERO_STEP;
 	}
-	return true;
+	L.phase = LANE_PROBE;
+	return MARCH_GOES_ON;
+}
+
+// what the render marches are given besides the ray
+struct MarchGrid {
+	Params P; const uint8_t* bitfield; SkipTable skip;
+	SRF_HD bool skipping() const { return skip.dist != nullptr && bitfield != nullptr; }
+};
+
+// occupancy_sampler.cu:738-797 — jitter the start, then step to the first occupied cell
+struct AdvanceMarch {
+	MarchGrid G; uint32_t n_rays, spp; srf_ray_payload* payloads;
+	struct Lane { MarchLane m; uint32_t i; };
+	struct Hit { SRF_HD MarchEnd operator()(MarchLane&, const Probe&) const { return MARCH_STOPPED; } };
+	SRF_HD uint32_t lanes() const { return n_rays; }
+	SRF_HD void finish(Lane& L, MarchEnd end) const {
+		srf_ray_payload& pl = payloads[L.i];
+		pl.t = L.m.t;
+		if (end != MARCH_STOPPED) pl.alive = 0;
+		L.m.phase = LANE_IDLE;
+	}
+	SRF_HD MarchEnd begin(Lane& L, uint32_t i) const {
+		L.i = i;
+		L.m.phase = LANE_IDLE;
+		const srf_ray_payload& pl = payloads[i];
+		if (!pl.alive) return MARCH_NO_RAY;
+		float t = pl.t;
+		t += ld_random_val01(spp, i * 786433u, 0) * calc_dt(G.P, t, G.P.cone_angle_constant);
+		march_start(L.m, ld3(pl.o), ld3(pl.d), t, G.skipping());
+		return MARCH_GOES_ON;
+	}
+	SRF_HD MarchEnd probe(Lane& L) const { return march_probe(L.m, G.P, G.bitfield, G.skip, G.skipping(), Hit()); }
+	SRF_HD MarchEnd steps(Lane& L) const { return march_steps(L.m, G.P); }
+};
+
+// occupancy_sampler.cu:799-863 — next n_steps occupied samples of a live ray.  A ray that leaves the box or ends on a
+// zero step before that keeps its old t and records how many samples it got; an occupied sample's own step is taken
+// whatever its size.
+struct CoordsMarch {
+	MarchGrid G; uint32_t n_rays, n_steps; srf_ray_payload* payloads; float* coords;
+	struct Lane { MarchLane m; uint32_t i, j; Vec3 wdir; };
+	struct Hit {
+		float* c; uint32_t* j; uint32_t n_steps; Vec3 wdir;
+		SRF_HD MarchEnd operator()(MarchLane& L, const Probe& s) const {
+			float* q = c + 7 * (size_t)*j;
+			st3(q, s.w); q[3] = s.dt; st3(q + 4, wdir);
+			++*j;
+			L.t += s.dt;
+			if (*j == n_steps) return MARCH_STOPPED;
+			L.phase = LANE_PROBE;
+			return MARCH_GOES_ON;
+		}
+	};
+	SRF_HD uint32_t lanes() const { return n_rays; }
+	SRF_HD void finish(Lane& L, MarchEnd end) const {
+		srf_ray_payload& pl = payloads[L.i];
+		if (end == MARCH_STOPPED) { pl.t = L.m.t; pl.n_steps = n_steps; }
+		else pl.n_steps = L.j;
+		L.m.phase = LANE_IDLE;
+	}
+	SRF_HD MarchEnd begin(Lane& L, uint32_t i) const {
+		L.i = i; L.j = 0;
+		L.m.phase = LANE_IDLE;
+		const srf_ray_payload& pl = payloads[i];
+		if (!pl.alive) return MARCH_NO_RAY;
+		const Vec3 d = ld3(pl.d);
+		L.wdir = warp_direction(d);
+		march_start(L.m, ld3(pl.o), d, pl.t, G.skipping());
+		return n_steps == 0 ? MARCH_STOPPED : MARCH_GOES_ON;
+	}
+	SRF_HD MarchEnd probe(Lane& L) const {
+		Hit hit; hit.c = coords + 7 * (size_t)L.i * n_steps; hit.j = &L.j; hit.n_steps = n_steps; hit.wdir = L.wdir;
+		return march_probe(L.m, G.P, G.bitfield, G.skip, G.skipping(), hit);
+	}
+	SRF_HD MarchEnd steps(Lane& L) const { return march_steps(L.m, G.P); }
+};
+
+// one ray from begin to finish, the phases in turn
+template <class March>
+SRF_HD void march_alone(const March& M, uint32_t i) {
+	typename March::Lane L;
+	MarchEnd end = M.begin(L, i);
+	while (end == MARCH_GOES_ON) end = L.m.phase == LANE_PROBE ? M.probe(L) : M.steps(L);
+	if (end != MARCH_NO_RAY) M.finish(L, end);
 }
 
 SRF_HD void advance_pos_body(uint32_t i, const Params& P, uint32_t spp, srf_ray_payload* payloads, const uint8_t* bitfield, SkipTable skip) {
-	srf_ray_payload& pl = payloads[i];
-	if (!pl.alive) return;
-	const Vec3 o = ld3(pl.o), d = ld3(pl.d);
-	const float cone = P.cone_angle_constant;
-	float t = pl.t;
-	t += ld_random_val01(spp, i * 786433u, 0) * calc_dt(P, t, cone);
-	const bool skipping = skip.dist != nullptr && bitfield != nullptr;
-	SkipRay sr;
-	if (skipping) sr = skip_ray_setup(o, d);
-	for (;;) {
-		const Vec3 pos = along(o, d, t);
-		if (!aabb_contains(P, pos)) { pl.alive = 0; break; }
-		const Probe s = probe_at(P, bitfield, pos, t, cone, &skip);
-		if (s.occ) break;
-		const float t_limit = skipping ? skip_limit(P, skip, sr, o, d, t, s.radius, s.level) : t;
-		t += s.dt;
-		if (s.dt == 0.f || !march_through_empty(P, t, t_limit, cone)) { pl.alive = 0; break; }
-	}
-	pl.t = t;
+	AdvanceMarch M;
+	M.G.P = P; M.G.bitfield = bitfield; M.G.skip = skip; M.n_rays = i + 1; M.spp = spp; M.payloads = payloads;
+	march_alone(M, i);
 }
 
-// occupancy_sampler.cu:799-863 — next n_steps occupied samples of a live ray
 SRF_HD void generate_coords_body(uint32_t i, const Params& P, uint32_t n_steps, const uint8_t* bitfield, srf_ray_payload* payloads, float* coords, SkipTable skip) {
-	srf_ray_payload& pl = payloads[i];
-	if (!pl.alive) return;
-	const Vec3 o = ld3(pl.o), d = ld3(pl.d);
-	const Vec3 wdir = warp_direction(d);
-	const float cone = P.cone_angle_constant;
-	float t = pl.t;
-	const bool skipping = skip.dist != nullptr && bitfield != nullptr;
-	SkipRay sr;
-	if (skipping) sr = skip_ray_setup(o, d);
-	for (uint32_t j = 0; j < n_steps; ++j) {
-		Probe s;
-		for (;;) {
-			const Vec3 pos = along(o, d, t);
-			if (!aabb_contains(P, pos)) { pl.n_steps = j; return; }
-			s = probe_at(P, bitfield, pos, t, cone, &skip);
-			if (s.occ) break;
-			const float t_limit = skipping ? skip_limit(P, skip, sr, o, d, t, s.radius, s.level) : t;
-			t += s.dt;
-			if (s.dt == 0.f || !march_through_empty(P, t, t_limit, cone)) { pl.n_steps = j; return; }
-		}
-		float* c = coords + 7 * ((size_t)i * n_steps + j);
-		st3(c, s.w); c[3] = s.dt; st3(c + 4, wdir);
-		t += s.dt;
-	}
-	pl.t = t;
-	pl.n_steps = n_steps;
+	CoordsMarch M;
+	M.G.P = P; M.G.bitfield = bitfield; M.G.skip = skip; M.n_rays = i + 1; M.n_steps = n_steps; M.payloads = payloads; M.coords = coords;
+	march_alone(M, i);
 }
 
 // ------------------------------------------------------------------------------------
@@ -896,58 +971,84 @@ SRF_HD void field_eval_body(uint32_t i, const Params& P, const float* coords, co
 	net_store<HALF>(out, (size_t)i * width + 3, row.w);
 }
 
-// Whole-frame render of pixel idx: the ray is generated, advanced and marched to the
+// Whole-frame render: the ray of a pixel is generated, advanced and marched to the
 // end, compositing every occupied sample as volume_rendering_kernel does
 // (ray_marcher.cu:233-273) and finishing with shade_kernel's store (testbed.cu:448-477)
 // into a frame buffer that starts from zero.  An occupied sample whose step size is
 // zero (t at the far plane, still inside the box) makes the reference's loop re-emit it
 // with zero weight until MARCH_ITER runs out (testbed.cu:523) and the still-alive ray is
 // never shaded; the pixel is left at zero here as well.
+// Lanes are numbered so that the 64 of a wavefront cover an 8 x 8 tile of pixels: neighbours in both directions take
+// similar paths through the grid.
+struct FusedMarch {
+	MarchGrid G; PixelArgs A; FieldArgs F; uint32_t spp; float thr; int to_linear; float* frame; uint32_t* n_samples;
+	struct Lane { MarchLane m; uint32_t idx, count; Float4 acc; };
+	struct Hit {
+		const Params* P; const FieldArgs* F; float thr; Float4* acc; uint32_t* count;
+		SRF_HD MarchEnd operator()(MarchLane& L, const Probe& s) const {
+			if (s.dt == 0.f) { *acc = mk4(0.f, 0.f, 0.f, 0.f); return MARCH_STOPPED; }
+			const Float4 row = *(const Float4*)(F->table + 4 * (size_t)field_row(*P, s.w, *F));
+			const float T = 1.f - acc->w;
+			const float alpha = 1.f - srf_expf(-row.w * s.dt);
+			const float weight = alpha * T;
+			acc->x += row.x * weight; acc->y += row.y * weight; acc->z += row.z * weight;
+			acc->w += weight;
+			++*count;
+			if (acc->w > (1.0f - thr)) return MARCH_STOPPED;
+			L.t += s.dt;
+			L.phase = LANE_PROBE;
+			return MARCH_GOES_ON;
+		}
+	};
+	SRF_HD uint32_t tiles_x() const { return ((uint32_t)A.res[0] + 7u) >> 3; }
+	SRF_HD uint32_t lanes() const { return tiles_x() * (((uint32_t)A.res[1] + 7u) >> 3) * 64u; }
+	SRF_HD void finish(Lane& L, MarchEnd) const {
+		Float4 out = mk4(0.f, 0.f, 0.f, 0.f);
+		if (L.acc.w > 0.001f) {
+			out = L.acc;
+			if (to_linear) { out.x = srgb_to_linear(out.x); out.y = srgb_to_linear(out.y); out.z = srgb_to_linear(out.z); }
+		}
+		*(Float4*)(frame + 4 * (size_t)L.idx) = out;
+		if (n_samples) n_samples[L.idx] = L.count;
+		L.m.phase = LANE_IDLE;
+	}
+	SRF_HD MarchEnd begin_pixel(Lane& L, uint32_t x, uint32_t y) const {
+		L.idx = x + (uint32_t)A.res[0] * y;
+		L.count = 0;
+		L.acc = mk4(0.f, 0.f, 0.f, 0.f);
+		Vec3 o, d;
+		pixel_ray(A, x, y, &o, &d);
+		float tmin, tmax;
+		aabb_ray_intersect(G.P, o, d, &tmin, &tmax);
+		float t = srf_max(tmin, 0.05f) + 1e-6f;
+		if (!aabb_contains(G.P, mk3(o.x + d.x * t, o.y + d.y * t, o.z + d.z * t))) return MARCH_LEFT_BOX;
+		t += ld_random_val01(spp, L.idx * 786433u, 0) * calc_dt(G.P, t, G.P.cone_angle_constant);
+		march_start(L.m, o, d, t, G.skipping());
+		return MARCH_GOES_ON;
+	}
+	SRF_HD MarchEnd begin(Lane& L, uint32_t q) const {
+		const uint32_t tile = q >> 6, tx = tiles_x();
+		const uint32_t x = (tile % tx) * 8u + (q & 7u), y = (tile / tx) * 8u + ((q >> 3) & 7u);
+		L.m.phase = LANE_IDLE;
+		return x < (uint32_t)A.res[0] && y < (uint32_t)A.res[1] ? begin_pixel(L, x, y) : MARCH_NO_RAY;
+	}
+	SRF_HD MarchEnd probe(Lane& L) const {
+		Hit hit; hit.P = &G.P; hit.F = &F; hit.thr = thr; hit.acc = &L.acc; hit.count = &L.count;
+		return march_probe(L.m, G.P, G.bitfield, G.skip, G.skipping(), hit);
+	}
+	SRF_HD MarchEnd steps(Lane& L) const { return march_steps(L.m, G.P); }
+};
+
 SRF_HD void render_fused_body(uint32_t idx, const Params& P, const PixelArgs& A, uint32_t spp, const uint8_t* bitfield, const FieldArgs& F,
                               float transmittance_threshold, int to_linear, float* frame, uint32_t* n_samples, SkipTable skip) {
-	const uint32_t x = idx % (uint32_t)A.res[0], y = idx / (uint32_t)A.res[0];
-	Vec3 o, d;
-	pixel_ray(A, x, y, &o, &d);
-	float tmin, tmax;
-	aabb_ray_intersect(P, o, d, &tmin, &tmax);
-	float t = srf_max(tmin, 0.05f) + 1e-6f;
-	Float4 acc = mk4(0.f, 0.f, 0.f, 0.f);
-	uint32_t count = 0;
-	if (aabb_contains(P, mk3(o.x + d.x * t, o.y + d.y * t, o.z + d.z * t))) {
-		const float cone = P.cone_angle_constant;
-		t += ld_random_val01(spp, idx * 786433u, 0) * calc_dt(P, t, cone);
-		const bool skipping = skip.dist != nullptr && bitfield != nullptr;
-		SkipRay sr;
-		if (skipping) sr = skip_ray_setup(o, d);
-		for (;;) {
-			const Vec3 pos = along(o, d, t);
-			if (!aabb_contains(P, pos)) break;
-			const Probe s = probe_at(P, bitfield, pos, t, cone, &skip);
-			float t_limit = t;
-			if (s.occ) {
-				if (s.dt == 0.f) { acc = mk4(0.f, 0.f, 0.f, 0.f); break; }
-				const Float4 row = *(const Float4*)(F.table + 4 * (size_t)field_row(P, s.w, F));
-				const float T = 1.f - acc.w;
-				const float alpha = 1.f - srf_expf(-row.w * s.dt);
-				const float weight = alpha * T;
-				acc.x += row.x * weight; acc.y += row.y * weight; acc.z += row.z * weight;
-				acc.w += weight;
-				++count;
-				if (acc.w > (1.0f - transmittance_threshold)) break;
-			} else if (skipping) {
-				t_limit = skip_limit(P, skip, sr, o, d, t, s.radius, s.level);
-			}
-			t += s.dt;
-			if (s.dt == 0.f || !march_through_empty(P, t, t_limit, cone)) break;
-		}
-	}
-	Float4 out = mk4(0.f, 0.f, 0.f, 0.f);
-	if (acc.w > 0.001f) {
-		out = acc;
-		if (to_linear) { out.x = srgb_to_linear(out.x); out.y = srgb_to_linear(out.y); out.z = srgb_to_linear(out.z); }
-	}
-	*(Float4*)(frame + 4 * (size_t)idx) = out;
-	if (n_samples) n_samples[idx] = count;
+	FusedMarch M;
+	M.G.P = P; M.G.bitfield = bitfield; M.G.skip = skip; M.A = A; M.F = F; M.spp = spp; M.thr = transmittance_threshold;
+	M.to_linear = to_linear; M.frame = frame; M.n_samples = n_samples;
+	FusedMarch::Lane L;
+	L.m.phase = LANE_IDLE;
+	MarchEnd end = M.begin_pixel(L, idx % (uint32_t)A.res[0], idx / (uint32_t)A.res[0]);
+	while (end == MARCH_GOES_ON) end = L.m.phase == LANE_PROBE ? M.probe(L) : M.steps(L);
+	M.finish(L, end);
 }
 
 // ------------------------------------------------------------------------------------

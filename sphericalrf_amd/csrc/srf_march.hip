@@ -233,16 +233,73 @@ __global__ void __launch_bounds__(128) k_init_rays(Params P, PixelArgs A, srf_ra
 	if (x < (uint32_t)A.res[0] && y < (uint32_t)A.res[1]) init_ray_body(x, y, P, A, payloads);
 }
 
-__global__ void __launch_bounds__(128) k_advance_pos(Params P, uint32_t n_rays, uint32_t spp, srf_ray_payload* __restrict__ payloads,
-                                                     const uint8_t* __restrict__ bitfield, SkipTable skip) {
-	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-	if (i < n_rays) advance_pos_body(i, P, spp, payloads, bitfield, skip);
+// The render marches (first occupied cell, next chunk of samples, whole frame), one wavefront per block and one ray per
+// lane.  Every round the wavefront runs one phase of srf_bodies.h's march machine: steps through known-empty space while
+// any lane has some to take, a grid probe (with whatever the march does at an occupied cell) once all lanes wait for one.
+// A lane waiting for its probe idles through the step rounds, so that the expensive probe is issued for all lanes at once.
+// Letting the probing lanes go first once they outnumber the stepping ones, and stepping in bursts of a fixed length (as the
+// counting march does), costs 5 to 15 % of a frame on the render workloads: here most lanes walk the same long empty
+// stretches side by side.
+#ifdef SRF_KERNEL_TIMING
+// per phase (step, probe): cycles, rounds, lanes that took part; then wavefronts, their lifetime in cycles, the longest in 10 ns ticks
+__device__ unsigned long long g_march_timing[16];
+#endif
+template <class March>
+__global__ void __launch_bounds__(64) k_march_lanes(March M) {
+	const uint32_t q = blockIdx.x * 64u + threadIdx.x;
+	typename March::Lane L;
+	L.m.phase = LANE_IDLE;
+#ifdef SRF_KERNEL_TIMING
+	unsigned long long t_acc_[6] = {0, 0, 0, 0, 0, 0};
+	unsigned long long t_prev_ = clock64();
+	const unsigned long long t_first_ = t_prev_, w_first_ = wall_clock64();
+#define SRF_MARCH_STAMP(k, lanes) do { const unsigned long long now_ = clock64(); t_acc_[k] += now_ - t_prev_; t_prev_ = now_; t_acc_[2 + k] += 1; t_acc_[4 + k] += (lanes); } while (0)
+#else
+#define SRF_MARCH_STAMP(k, lanes) ((void)0)
+#endif
+	// a lane's march ends in begin, probe or steps; its results are stored in one place, here
+	MarchEnd end = q < M.lanes() ? M.begin(L, q) : MARCH_NO_RAY;
+	for (;;) {
+		if (end != MARCH_GOES_ON) {
+			if (end != MARCH_NO_RAY) M.finish(L, end);
+			L.m.phase = LANE_IDLE;
+			end = MARCH_GOES_ON;
+		}
+		const uint32_t n_probe = (uint32_t)__popcll(__ballot(L.m.phase == LANE_PROBE));
+		const uint32_t n_step = (uint32_t)__popcll(__ballot(L.m.phase == LANE_STEP));
+		if (!(n_probe | n_step)) break;
+		if (n_step) {
+			if (L.m.phase == LANE_STEP) end = M.steps(L);
+			SRF_MARCH_STAMP(0, n_step);
+		} else {
+			if (L.m.phase == LANE_PROBE) end = M.probe(L);
+			SRF_MARCH_STAMP(1, n_probe);
+		}
+	}
+#ifdef SRF_KERNEL_TIMING
+	if (threadIdx.x == 0) {
+		for (int k = 0; k < 6; ++k) atomicAdd(&g_march_timing[k], t_acc_[k]);
+		atomicAdd(&g_march_timing[6], 1ull);
+		atomicAdd(&g_march_timing[7], clock64() - t_first_);
+		atomicMax(&g_march_timing[8], wall_clock64() - w_first_);
+	}
+#endif
 }
 
-__global__ void __launch_bounds__(128) k_generate_coords(Params P, uint32_t n_rays, uint32_t n_steps, const uint8_t* __restrict__ bitfield,
-                                                         srf_ray_payload* __restrict__ payloads, float* __restrict__ coords, SkipTable skip) {
-	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-	if (i < n_rays) generate_coords_body(i, P, n_steps, bitfield, payloads, coords, skip);
+template <class March>
+static void launch_march(const March& M, hipStream_t st) {
+	hipLaunchKernelGGL(k_march_lanes<March>, dim3(div_up(M.lanes(), 64u)), dim3(64), 0, st, M);
+#ifdef SRF_KERNEL_TIMING
+	unsigned long long h[16], zero[16] = {0};
+	if (hipStreamSynchronize(st) != hipSuccess || hipMemcpyFromSymbol(h, HIP_SYMBOL(g_march_timing), sizeof(h)) != hipSuccess) return;
+	(void)hipMemcpyToSymbol(HIP_SYMBOL(g_march_timing), zero, sizeof(zero));
+	const double nw = (double)(h[6] ? h[6] : 1);
+	fprintf(stderr, "march of %u lanes: wavefront lifetime %.0f cycles mean, %.1f us longest\n", M.lanes(), (double)h[7] / nw, (double)h[8] / 100.0);
+	const char* name[2] = {"step", "probe"};
+	for (int k = 0; k < 2; ++k)
+		fprintf(stderr, "march %-5s: %.0f cycles per wavefront, %.1f rounds, %.0f cycles per round, %.1f lanes per round\n", name[k],
+		        (double)h[k] / nw, (double)h[2 + k] / nw, h[2 + k] ? (double)h[k] / (double)h[2 + k] : 0.0, h[2 + k] ? (double)h[4 + k] / (double)h[2 + k] : 0.0);
+#endif
 }
 
 template <bool HALF>
@@ -251,16 +308,17 @@ __global__ void __launch_bounds__(256) k_field_eval(Params P, uint32_t n, const 
 	if (i < n) field_eval_body<HALF>(i, P, coords, F, out, width);
 }
 
-__global__ void __launch_bounds__(128) k_render_fused(Params P, PixelArgs A, uint32_t spp, const uint8_t* __restrict__ bitfield, FieldArgs F,
-                                                      float transmittance_threshold, int to_linear,
-                                                      float* __restrict__ frame, uint32_t* __restrict__ n_samples, SkipTable skip) {
-	const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
-	if (idx < (uint32_t)A.res[0] * (uint32_t)A.res[1]) render_fused_body(idx, P, A, spp, bitfield, F, transmittance_threshold, to_linear, frame, n_samples, skip);
-}
-
 // the sampler's empty-space table when it matches the bitfield, an empty one otherwise
 static SkipTable sampler_skip_table(const srf_sampler* s) {
 	return skip_table_for(s->P, s->skip_valid ? s->skip_dist : nullptr);
+}
+
+static MarchGrid sampler_march_grid(const srf_sampler* s) {
+	MarchGrid G;
+	G.P = s->P;
+	G.bitfield = s->P.use_grid ? s->density_grid_bitfield : nullptr;
+	G.skip = sampler_skip_table(s);
+	return G;
 }
 
 static void fill_pixel_args(PixelArgs& A, const Params& P, const int32_t resolution[2], const float focal_length[2],
@@ -426,8 +484,9 @@ int srf_sampler_generate_rays_from_camera_matrix(srf_sampler_t* s, const int32_t
 	hipLaunchKernelGGL(k_init_rays, blocks, threads, 0, st, s->P, A, payload);
 	SRF_LAUNCH_CHECK();
 	const uint32_t n = (uint32_t)resolution[0] * (uint32_t)resolution[1];
-	hipLaunchKernelGGL(k_advance_pos, dim3(div_up(n, 128)), dim3(128), 0, st, s->P, n, spp, payload,
-	                   (const uint8_t*)(s->P.use_grid ? s->density_grid_bitfield : nullptr), sampler_skip_table(s));
+	AdvanceMarch M;
+	M.G = sampler_march_grid(s); M.n_rays = n; M.spp = spp; M.payloads = payload;
+	launch_march(M, st);
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }
@@ -437,8 +496,9 @@ int srf_sampler_generate_coords_from_rays(srf_sampler_t* s, uint32_t n_rays, uin
 	SRF_REQUIRE(s, "srf_sampler_generate_coords_from_rays: NULL sampler");
 	if (n_rays == 0 || n_steps == 0) return SRF_OK;
 	SRF_REQUIRE(payloads && coords, "srf_sampler_generate_coords_from_rays: NULL buffer");
-	hipLaunchKernelGGL(k_generate_coords, dim3(div_up(n_rays, 128)), dim3(128), 0, (hipStream_t)stream, s->P, n_rays, n_steps,
-	                   (const uint8_t*)(s->P.use_grid ? s->density_grid_bitfield : nullptr), payloads, coords, sampler_skip_table(s));
+	CoordsMarch M;
+	M.G = sampler_march_grid(s); M.n_rays = n_rays; M.n_steps = n_steps; M.payloads = payloads; M.coords = coords;
+	launch_march(M, (hipStream_t)stream);
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }
@@ -471,11 +531,12 @@ int srf_render_frame_fused(srf_sampler_t* s, const srf_marcher_t* m, const srf_f
 	SRF_REQUIRE(s->P.griddist_type == SRF_GRID_WARPED_EXP || s->P.griddist_type == SRF_GRID_WARPED_RECIPROCAL, "srf_render_frame_fused: needs a warped-space grid type");
 	PixelArgs A;
 	fill_pixel_args(A, s->P, resolution, focal_length, principal_point, camera_matrix_host, spp);
-	FieldArgs F; F.table = field->table; F.mask = field->table_size - 1; F.seed = field->seed;
-	const uint32_t n = (uint32_t)resolution[0] * (uint32_t)resolution[1];
-	hipLaunchKernelGGL(k_render_fused, dim3(div_up(n, 128)), dim3(128), 0, (hipStream_t)stream, s->P, A, spp,
-	                   (const uint8_t*)(s->P.use_grid ? s->density_grid_bitfield : nullptr), F,
-	                   m->cfg.transmittance_threshold, m->cfg.train_in_linear_color ? 0 : 1, frame_buffer, n_samples, sampler_skip_table(s));
+	FusedMarch M;
+	M.G = sampler_march_grid(s); M.A = A; M.spp = spp;
+	M.F.table = field->table; M.F.mask = field->table_size - 1; M.F.seed = field->seed;
+	M.thr = m->cfg.transmittance_threshold; M.to_linear = m->cfg.train_in_linear_color ? 0 : 1;
+	M.frame = frame_buffer; M.n_samples = n_samples;
+	launch_march(M, (hipStream_t)stream);
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }
