@@ -144,6 +144,15 @@ int  srf_sampler_set_runtime(srf_sampler_t* s, int32_t snap_train, int32_t snap_
 int  srf_sampler_init(srf_sampler_t* s, uint32_t n_images, const int32_t image_resolution[2], const float focal_length[2],
                       const float principal_point[2], const float* camera_matrices, srf_pcg32* rng_host, void* stream);
 
+/* No counterpart in the reference, which bounds rays by the box alone (bounding_box.h:145-180); off unless set.  With a
+ * sphere set, the training and render marches keep exactly those samples of the unbounded march whose t lies within the
+ * ray's stretch inside the sphere (the chain of t is not moved); radius <= 0 removes the bound.  Takes effect from the next call. */
+int  srf_sampler_set_ray_sphere_bound(srf_sampler_t* s, const float center[3], float radius);
+
+/* The same stretch for n_rays rays laid out as (origin, direction) x 6 floats: t_near[i] <= t <= t_far[i] is inside the
+ * sphere; a ray whose line misses it gets t_near = +inf, t_far = -inf.  All pointers device memory. */
+int  srf_ray_sphere_bounds(uint32_t n_rays, const float* rays, const float center[3], float radius, float* t_near, float* t_far, void* stream);
+
 /* Testbed::load_snapshot, internal/testbed.cu:167: overwrite density_grid (n_total_elements floats, device) */
 int  srf_sampler_set_density_grid(srf_sampler_t* s, const float* density_grid, void* stream);
 

@@ -252,6 +252,11 @@ class OccupancySampler:
                                          C.byref((K.f32 * 2)(*principal_point)), _dev(camera_matrices, allow_none=True), C.byref(r), _stream()))
         rng.state, rng.inc = r.state, r.inc
 
+    def set_ray_sphere_bound(self, center, radius):
+        """bounds the marches by a sphere as well (no counterpart in the reference; radius <= 0 removes the bound): exactly those
+        samples of the unbounded march remain whose t lies within the ray's stretch inside the sphere"""
+        K.check(self._L.srf_sampler_set_ray_sphere_bound(self._h, C.byref((K.f32 * 3)(*[float(v) for v in center])), float(radius)))
+
     def set_density_grid(self, grid):
         K.check(self._L.srf_sampler_set_density_grid(self._h, _dev(grid, torch.float32, self.info.n_total_elements, "grid"), _stream()))
 
@@ -330,6 +335,13 @@ class OccupancySampler:
         K.check(self._L.srf_render_frame(self._h, marcher._h, C.byref(a), fn, user, _dev(frame_buffer, torch.float32, 4 * n, "frame_buffer"), C.byref(iters), _stream()))
         del keep
         return int(iters.value)
+
+
+def ray_sphere_bounds(rays, center, radius, t_near, t_far):
+    """the stretch t_near <= t <= t_far of every ray (origin, direction: 6 floats) inside a sphere; (+inf, -inf) for a miss"""
+    n = rays.numel() // 6
+    K.check(K.load().srf_ray_sphere_bounds(n, _dev(rays, torch.float32, 6 * n, "rays"), C.byref((K.f32 * 3)(*[float(v) for v in center])), float(radius),
+                                           _dev(t_near, torch.float32, n, "t_near"), _dev(t_far, torch.float32, n, "t_far"), _stream()))
 
 
 def frame_accumulate(resolution, frame_buffer, accumulate_buffer, spp, color_space=K.COLOR_LINEAR):

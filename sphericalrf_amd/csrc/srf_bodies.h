@@ -417,9 +417,22 @@ SRF_HD void count_unpark(CountLane& L, const ParkedRay& r) {
 }
 
 // occupancy_sampler.cu:595-628 — a step that looks its cell up
+// SPHERE = false compiles the optional sphere bound out (the counting kernel is short of registers; it is built both ways)
+template <bool SPHERE = true>
 SRF_HD void count_probe(CountLane& L, const Params& P, const CountArgs& A) {
 	const Vec3 pos = along(L.o, L.d, L.t);
 	if (!(aabb_contains(P, pos) && L.j < P.n_max_steps)) { count_finish(L, A); return; }
+	if (SPHERE && P.sphere[3] > 0.f) {      // optional sphere bound: no sample outside it, the chain of t as it is
+		float t_enter;
+		const SphereGate g = sphere_gate(P, L.o, L.d, L.t, &t_enter);
+		if (g == SPHERE_BEYOND) { count_finish(L, A); return; }
+		if (g == SPHERE_BEFORE) {
+			L.t_limit = t_enter;
+			count_advance(L, A, calc_dt(P, L.t, P.cone_angle_constant));
+			if (L.phase != LANE_IDLE) L.phase = L.t < L.t_limit ? LANE_STEP : LANE_PROBE;
+			return;
+		}
+	}
 	if (A.probe_budget && L.probes >= A.probe_budget && count_park(L, A)) return;
 	++L.probes;
 	SRF_COUNT_PROBE();
@@ -564,6 +577,12 @@ SRF_HD WideLookup wide_lookup(const Params& P, const CountArgs& A, Vec3 o, Vec3 
 	const Vec3 pos = along(o, d, t);
 	q.inside = aabb_contains(P, pos);
 	q.byte = 0xffu; q.bit = 0u;
+	if (q.inside && P.sphere[3] > 0.f) {
+		float t_enter;
+		const SphereGate g = sphere_gate(P, o, d, t, &t_enter);
+		if (g == SPHERE_BEYOND) q.inside = false;
+		if (g == SPHERE_BEFORE) { q.byte = 0u; return q; }
+	}
 	if (q.inside && P.use_grid) {
 		const Probe s = probe_at(P, nullptr, pos, t, P.cone_angle_constant);   // the cell only
 		q.bit = s.idx & 7u;
@@ -738,6 +757,17 @@ SRF_HD void train_write_march(const Params& P, const uint8_t* bitfield, const Wr
 	for (;;) {
 		const Vec3 pos = along(R.o, R.d, t);
 		if (!(aabb_contains(P, pos) && j < cap)) break;
+		if (P.sphere[3] > 0.f) {
+			float t_enter;
+			const SphereGate g = sphere_gate(P, R.o, R.d, t, &t_enter);
+			if (g == SPHERE_BEYOND) break;
+			if (g == SPHERE_BEFORE) {
+				const float dt = calc_dt(P, t, cone);
+				t += dt;
+				if (dt == 0.f) break;
+				continue;
+			}
+		}
 		const Probe s = probe_at(P, P.use_grid ? bitfield : nullptr, pos, t, cone);
 		if (s.occ) {
 			const size_t k = (size_t)R.base + j;
@@ -823,6 +853,19 @@ SRF_HD MarchEnd march_probe(MarchLane& L, const Params& P, const uint8_t* bitfie
 	const float cone = P.cone_angle_constant;
 	const Vec3 pos = along(L.o, L.d, L.t);
 	if (!aabb_contains(P, pos)) return MARCH_LEFT_BOX;
+	if (P.sphere[3] > 0.f) {      // optional sphere bound: no sample outside it, the chain of t as it is
+		float t_enter;
+		const SphereGate g = sphere_gate(P, L.o, L.d, L.t, &t_enter);
+		if (g == SPHERE_BEYOND) return MARCH_LEFT_BOX;
+		if (g == SPHERE_BEFORE) {
+			const float dt = calc_dt(P, L.t, cone);
+			L.t_limit = t_enter;
+			L.t += dt;
+			if (dt == 0.f) return MARCH_ZERO_STEP;
+			L.phase = L.t < L.t_limit ? LANE_STEP : LANE_PROBE;
+			return MARCH_GOES_ON;
+		}
+	}
 	const Probe s = probe_at(P, bitfield, pos, L.t, cone, &skip);
 	L.t_limit = L.t;      // steps at t' < t_limit are known to find an empty cell
 	if (s.occ) return hit(L, s);

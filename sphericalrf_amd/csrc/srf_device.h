@@ -38,6 +38,7 @@ struct Params {
 	float    min_optical_thickness;
 	float    ema_decay;
 	uint32_t n_cells;          // grid_size[0]*grid_size[1]*grid_size[2]
+	float    sphere[4];        // optional bound of the marches: centre and radius, radius <= 0 = none (not in the reference)
 };
 
 struct Vec3 { float x, y, z; };
@@ -266,6 +267,32 @@ SRF_HD void aabb_ray_intersect(const Params& P, Vec3 o, Vec3 d, float* tmin_out,
 SRF_HD bool aabb_contains(const Params& P, Vec3 p) {
 	return p.x >= P.aabb_min[0] && p.x <= P.aabb_max[0] && p.y >= P.aabb_min[1] && p.y <= P.aabb_max[1] &&
 	       p.z >= P.aabb_min[2] && p.z <= P.aabb_max[2];
+}
+
+// The stretch [t0, t1] of a ray inside a sphere, from the quadratic |o + t d - c|^2 = r^2 written around the ray's closest
+// approach: t_mid = -(m.d)/(d.d), half = sqrt((m.d)^2 - (d.d)(m.m - r^2))/(d.d), m = o - c.  A ray whose line misses the
+// sphere (or a direction of length zero) has no stretch.  Not in the reference, which bounds rays by the box alone.
+struct SphereSpan { float t0, t1; bool hit; };
+SRF_HD SphereSpan sphere_ray_span(const float sphere[4], Vec3 o, Vec3 d) {
+	const Vec3 m = sub3(o, ld3(sphere));
+	const float a = dot3(d, d), b = dot3(m, d), c = dot3(m, m) - sphere[3] * sphere[3];
+	const float disc = b * b - a * c;
+	SphereSpan sp;
+	sp.hit = a > 0.f && disc >= 0.f;
+	sp.t0 = sp.t1 = 0.f;
+	if (sp.hit) {
+		const float half = srf_sqrt(disc) / a, mid = -b / a;
+		sp.t0 = mid - half; sp.t1 = mid + half;
+	}
+	return sp;
+}
+// where a march at t stands against the optional sphere: before it (nothing to find until *t_enter), inside, or past it for good
+enum SphereGate : uint32_t { SPHERE_INSIDE = 0, SPHERE_BEFORE = 1, SPHERE_BEYOND = 2 };
+SRF_HD SphereGate sphere_gate(const Params& P, Vec3 o, Vec3 d, float t, float* t_enter) {
+	const SphereSpan sp = sphere_ray_span(P.sphere, o, d);
+	if (!sp.hit || t > sp.t1) return SPHERE_BEYOND;
+	if (t < sp.t0) { *t_enter = sp.t0; return SPHERE_BEFORE; }
+	return SPHERE_INSIDE;
 }
 
 // ------------------------------------------------------------------------------------

@@ -50,6 +50,7 @@ __global__ void __launch_bounds__(RAY_CHUNK_BINS) k_ray_order(Params P, CountArg
 	for (uint32_t j = threadIdx.x; j < n; j += RAY_CHUNK_BINS) order[first + atomicAdd(&bins[keys[j]], 1u)] = first + j;
 }
 
+template <bool SPHERE>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(SRF_COUNT_WAVES_PER_EU))) k_train_count(Params P, CountArgs A, uint32_t rays_per_wave, uint32_t probe_quorum, uint32_t begin_quorum, uint32_t probe_ratio,
                                                                                                                     const uint32_t* __restrict__ order, unsigned long long* timing) {
 	const uint32_t lane = threadIdx.x;
@@ -82,7 +83,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(SRF_COU
 			if (L.phase == LANE_STEP) count_steps<COUNT_STEP_BURST>(L, P, A);
 			SRF_COUNT_STAMP(0, n_step);
 		} else if (!begin) {
-			if (L.phase == LANE_PROBE) count_probe(L, P, A);
+			if (L.phase == LANE_PROBE) count_probe<SPHERE>(L, P, A);
 			SRF_COUNT_STAMP(1, n_probe);
 		} else {
 			const uint32_t rank = (uint32_t)__popcll(m_idle & ((1ull << lane) - 1ull));
@@ -302,6 +303,16 @@ static void launch_march(const March& M, hipStream_t st) {
 #endif
 }
 
+// the stretch of every ray inside a sphere; a ray that misses it gets the empty stretch (+inf, -inf).  24 B in, 8 B out a ray.
+__global__ void __launch_bounds__(256) k_ray_sphere_bounds(uint32_t n_rays, const float* __restrict__ rays, Float4 sphere, float* __restrict__ t_near, float* __restrict__ t_far) {
+	const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+	if (i >= n_rays) return;
+	const float c[4] = {sphere.x, sphere.y, sphere.z, sphere.w};
+	const SphereSpan sp = sphere_ray_span(c, ld3(rays + 6 * (size_t)i), ld3(rays + 6 * (size_t)i + 3));
+	t_near[i] = sp.hit ? sp.t0 : srf_u2f(0x7f800000u);
+	t_far[i] = sp.hit ? sp.t1 : srf_u2f(0xff800000u);
+}
+
 template <bool HALF>
 __global__ void __launch_bounds__(256) k_field_eval(Params P, uint32_t n, const float* __restrict__ coords, FieldArgs F, void* __restrict__ out, uint32_t width) {
 	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -422,7 +433,10 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 	if (!timing_buf) { SRF_HIP(hipMalloc((void**)&timing_buf, (1024 * 16 + 192) * 8)); SRF_HIP(hipMemset(timing_buf, 0, (1024 * 16 + 192) * 8)); }
 	timing = timing_buf;
 #endif
-	hipLaunchKernelGGL(k_train_count, dim3(div_up(n_rays, rays_per_wave)), dim3(64), 0, st, s->P, ca, rays_per_wave, probe_quorum, begin_quorum, probe_ratio, order, timing);
+	if (s->P.sphere[3] > 0.f)
+		hipLaunchKernelGGL(k_train_count<true>, dim3(div_up(n_rays, rays_per_wave)), dim3(64), 0, st, s->P, ca, rays_per_wave, probe_quorum, begin_quorum, probe_ratio, order, timing);
+	else
+		hipLaunchKernelGGL(k_train_count<false>, dim3(div_up(n_rays, rays_per_wave)), dim3(64), 0, st, s->P, ca, rays_per_wave, probe_quorum, begin_quorum, probe_ratio, order, timing);
 #ifdef SRF_KERNEL_TIMING
 	{
 		static unsigned long long hs[1024 * 16 + 192];
@@ -467,6 +481,25 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 	hipLaunchKernelGGL(k_train_write, dim3(div_up(n_rays, 64)), dim3(64), 0, st, s->P, n_rays, ds, bitfield, (const TrainRay*)state,
 	                   (const uint32_t*)counts, (const uint32_t*)base, (const uint32_t*)keep, (const uint32_t*)ridx,
 	                   rays, rays_rgba, ray_coord_indices, coords, sample_t, sample_dt, sample_cell, log);
+	SRF_LAUNCH_CHECK();
+	return SRF_OK;
+}
+
+int srf_sampler_set_ray_sphere_bound(srf_sampler_t* s, const float center[3], float radius) {
+	SRF_REQUIRE(s, "srf_sampler_set_ray_sphere_bound: NULL sampler");
+	SRF_REQUIRE(radius <= 0.f || center, "srf_sampler_set_ray_sphere_bound: NULL center");
+	SRF_REQUIRE(radius == radius && radius < 3.0e38f, "srf_sampler_set_ray_sphere_bound: radius must be finite");
+	for (int a = 0; a < 3; ++a) s->P.sphere[a] = radius > 0.f ? center[a] : 0.f;
+	s->P.sphere[3] = radius > 0.f ? radius : 0.f;
+	return SRF_OK;
+}
+
+int srf_ray_sphere_bounds(uint32_t n_rays, const float* rays, const float center[3], float radius, float* t_near, float* t_far, void* stream) {
+	SRF_REQUIRE(center && radius > 0.f, "srf_ray_sphere_bounds: needs a center and a positive radius");
+	if (n_rays == 0) return SRF_OK;
+	SRF_REQUIRE(rays && t_near && t_far, "srf_ray_sphere_bounds: NULL buffer");
+	hipLaunchKernelGGL(k_ray_sphere_bounds, dim3(div_up(n_rays, 256)), dim3(256), 0, (hipStream_t)stream, n_rays, rays,
+	                   mk4(center[0], center[1], center[2], radius), t_near, t_far);
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }

@@ -18,12 +18,16 @@ static uint64_t g_radius_hist[8][4] = {};   // [cascade][radius 0, 1-block, 2-3,
 using namespace srf;
 
 static_assert(sizeof(srf_ray_payload) == 40, "payload layout");
-static_assert(sizeof(orc_params) + sizeof(uint32_t) == sizeof(Params), "Params mirrors orc_params plus n_cells");
+static_assert(sizeof(orc_params) + sizeof(uint32_t) + 4 * sizeof(float) == sizeof(Params), "Params mirrors orc_params plus n_cells and the optional sphere");
+
+// the optional sphere bound of the marches (the reference and the oracle have none): set by hs_set_sphere for the calls that follow
+static float g_sphere[4] = {0.f, 0.f, 0.f, 0.f};
 
 static Params to_params(const orc_params* p) {
 	Params P;
 	std::memcpy(&P, p, sizeof(orc_params));
 	P.n_cells = p->grid_size[0] * p->grid_size[1] * p->grid_size[2];
+	for (int k = 0; k < 4; ++k) P.sphere[k] = g_sphere[k];
 	return P;
 }
 
@@ -439,6 +443,16 @@ uint32_t hs_pcg_skip_mismatches(uint32_t seed, uint32_t n_cases) {
 		bad += a.state != b.state || a.inc != b.inc || a.state != h.state || a.inc != h.inc;
 	}
 	return bad;
+}
+
+void hs_set_sphere(const float sphere[4]) { for (int k = 0; k < 4; ++k) g_sphere[k] = sphere ? sphere[k] : 0.f; }
+
+// stretch of n rays (origin, direction) inside a sphere; hit[i] = 0 for a miss
+void hs_sphere_spans(uint32_t n, const float* rays, const float sphere[4], float* t0, float* t1, uint8_t* hit) {
+	for (uint32_t i = 0; i < n; ++i) {
+		const SphereSpan sp = sphere_ray_span(sphere, ld3(rays + 6 * (size_t)i), ld3(rays + 6 * (size_t)i + 3));
+		t0[i] = sp.t0; t1[i] = sp.t1; hit[i] = sp.hit ? 1 : 0;
+	}
 }
 
 // the reciprocal that the disparity chain carries: for how many of the 2^23 mantissas of g does one fused Newton step
