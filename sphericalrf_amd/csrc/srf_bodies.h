@@ -6,7 +6,7 @@
 #include "srf_device.h"
 #include "srf_skip.h"
 
-// hook for host builds that count how many steps of the training march probe the grid
+// hook for host builds that count how many steps of a march probe the grid
 #ifndef SRF_COUNT_PROBE
 #define SRF_COUNT_PROBE() ((void)0)
 #endif
@@ -866,6 +866,7 @@ SRF_HD MarchEnd march_probe(MarchLane& L, const Params& P, const uint8_t* bitfie
 			return MARCH_GOES_ON;
 		}
 	}
+	SRF_COUNT_PROBE();
 	const Probe s = probe_at(P, bitfield, pos, L.t, cone, &skip);
 	L.t_limit = L.t;      // steps at t' < t_limit are known to find an empty cell
 	if (s.occ) return hit(L, s);

@@ -36,7 +36,10 @@ SRF_HD uint32_t skip_blocks_per_axis(const Params& P) {
 	if (P.warping_type != SRF_WARP_ERP && P.warping_type != SRF_WARP_SINUSOIDAL) return 0;
 	const uint32_t gz = P.grid_size[2];
 	if (gz < 16) return 0;
-	const uint32_t nb = gz / 4;
+	// blocks of four cells a side; two on small grids, where the coarser table leaves most probes of a ray that runs through
+	// occupied surroundings in place (workload 1: 501 of 512 lookups a ray against 103) -- on a 128-grid the finer, 8 x larger
+	// table saves a seventh of the lookups and makes a frame a fifth slower
+	const uint32_t nb = gz <= 64 ? gz / 2 : gz / 4;
 	return nb < SKIP_MAX_BLOCKS ? nb : SKIP_MAX_BLOCKS;
 }
 
