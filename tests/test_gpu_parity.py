@@ -484,6 +484,27 @@ def test_every_loss_function(gpu, orc, loss, impl, monkeypatch):
     assert np.abs(o_dloss).max() > 0
 
 
+@pytest.mark.parametrize("res", [(37, 21), (8, 8), (9, 70), (131, 5), (1, 1)])
+def test_fused_frame_sizes_that_do_not_fill_their_pixel_tiles(gpu, orc, res):
+    """the fused frame hands 8 x 8 pixel tiles to its wavefronts: widths and heights that leave tiles partly outside the frame"""
+    torch = gpu
+    from sphericalrf_amd import api, scene
+    w, p, grid, bf, mean = helpers.build_scene(orc, 1, 0.5)
+    s = make_sampler(torch, api, w, grid)
+    m = api.RayMarcher(dict(train_in_linear_color=False, transmittance_threshold=1e-4))
+    f, cam = (scene.focal_from_fov(max(res), 60.0),) * 2, w["cameras"][-1]
+    table = scene.field_table(4096, 5)
+    table[:, 3] *= 20
+    want_frame, want_ns, _ = orc.render_frame(p, orc.make_field(table, 77), bf, res, f, (0.5, 0.5), cam, transmittance_threshold=1e-4, train_in_linear_colors=False)
+    n = res[0] * res[1]
+    guard = 64
+    frame = torch.full((n + guard, 4), 7.0, device="cuda")           # room behind the frame that must stay untouched
+    ns = torch.full((n + guard,), 9, dtype=torch.int32, device="cuda")
+    s.render_frame_fused(m, api.Field(torch.from_numpy(table).cuda(), 77), res, f, (0.5, 0.5), cam, frame, ns)
+    assert np.array_equal(u32(ns)[:n].reshape(res[1], res[0]), want_ns) and (u32(ns)[n:] == 9).all()
+    assert np.array_equal(frame.cpu().numpy()[:n].reshape(res[1], res[0], 4), want_frame) and (frame.cpu().numpy()[n:] == 7.0).all()
+
+
 @pytest.mark.parametrize("config_id,scale", [(1, 0.5), (2, 0.25), (2, 1.0), (3, 0.125)])
 def test_render_loop_and_fused_frame(gpu, orc, config_id, scale):
     """a frame through the fused kernel and through the reference's loop of entry points, against the oracle's frame; (2, 1.0) is
