@@ -618,31 +618,79 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 #endif
 }
 
-// testbed.cu:423-446 — classification of a ray: 1 alive, 2 finished with visible alpha, 0 dropped
-__global__ void __launch_bounds__(256) k_compact_flags(uint32_t n, const srf_ray_payload* __restrict__ payloads, const float* __restrict__ rgba,
-                                                       uint32_t* __restrict__ alive, uint32_t* __restrict__ fin) {
-	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-	if (i >= n) return;
-	const bool a = payloads[i].alive != 0;
-	alive[i] = a ? 1u : 0u;
-	fin[i] = (!a && rgba[4 * (size_t)i + 3] > 0.001f) ? 1u : 0u;
-}
-
+// testbed.cu:423-446 — compaction of the live rays into dst and of the finished, visible ones into the final buffers.
+// The reference hands positions out with one atomicAdd a ray, in whatever order the threads arrive; here the order is the
+// source order (every later stage then sees the same arrays run after run): blocks of 1024 rays count their two classes with
+// wave ballots (k_compact_count), and the moving kernel gives every block the sum of the counts before it (a block reads the
+// at most few thousand counts itself), every wavefront its offset inside the block, and every lane its rank from the ballot.
+constexpr uint32_t COMPACT_BLOCK = 1024;
 struct Payload40 { uint32_t w[10]; };
 
-__global__ void __launch_bounds__(256) k_compact_move(uint32_t n, const srf_ray_payload* __restrict__ src_p, const float* __restrict__ src_c,
-                                                      srf_ray_payload* __restrict__ dst_p, float* __restrict__ dst_c,
-                                                      srf_ray_payload* __restrict__ fin_p, float* __restrict__ fin_c,
-                                                      const uint32_t* __restrict__ alive, const uint32_t* __restrict__ alive_pos,
-                                                      const uint32_t* __restrict__ fin, const uint32_t* __restrict__ fin_pos) {
-	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-	if (i >= n) return;
-	if (alive[i]) {
-		const uint32_t k = alive_pos[i];
+// 1: alive, 2: finished with visible alpha, 0: dropped
+__device__ __forceinline__ uint32_t compact_class(uint32_t i, uint32_t n, const srf_ray_payload* __restrict__ payloads, const float* __restrict__ rgba) {
+	if (i >= n) return 0u;
+	if (payloads[i].alive != 0) return 1u;
+	return rgba[4 * (size_t)i + 3] > 0.001f ? 2u : 0u;
+}
+
+// counts[b] = {alive, finished} of block b; block 0 also notes the counters' values on entry, which are where this call's output starts
+__global__ void __launch_bounds__(COMPACT_BLOCK) k_compact_count(uint32_t n, const srf_ray_payload* __restrict__ payloads, const float* __restrict__ rgba,
+                                                                 U2* __restrict__ counts, const uint32_t* __restrict__ n_alive_counter,
+                                                                 const uint32_t* __restrict__ n_final_counter, uint32_t* __restrict__ initial, bool alive_from_zero) {
+	__shared__ uint32_t part[2][COMPACT_BLOCK / 64];
+	const uint32_t i = blockIdx.x * COMPACT_BLOCK + threadIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+	const uint32_t c = compact_class(i, n, payloads, rgba);
+	const uint32_t na = (uint32_t)__popcll(__ballot(c == 1u)), nf = (uint32_t)__popcll(__ballot(c == 2u));
+	if (lane == 0) { part[0][wave] = na; part[1][wave] = nf; }
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		uint32_t a = 0, f = 0;
+		for (uint32_t k = 0; k < COMPACT_BLOCK / 64; ++k) { a += part[0][k]; f += part[1][k]; }
+		U2 v; v.x = a; v.y = f;
+		counts[blockIdx.x] = v;
+		if (blockIdx.x == 0) { initial[0] = alive_from_zero ? 0u : *n_alive_counter; initial[1] = *n_final_counter; }
+	}
+}
+
+__global__ void __launch_bounds__(COMPACT_BLOCK) k_compact_move(uint32_t n, const srf_ray_payload* __restrict__ src_p, const float* __restrict__ src_c,
+                                                                srf_ray_payload* __restrict__ dst_p, float* __restrict__ dst_c,
+                                                                srf_ray_payload* __restrict__ fin_p, float* __restrict__ fin_c,
+                                                                const U2* __restrict__ counts, const uint32_t* __restrict__ initial,
+                                                                uint32_t* __restrict__ n_alive_counter, uint32_t* __restrict__ n_final_counter,
+                                                                unsigned long long* __restrict__ host_word, uint32_t stamp) {
+	__shared__ uint32_t part[2][COMPACT_BLOCK / 64];
+	__shared__ uint32_t before[2][COMPACT_BLOCK / 64];
+	__shared__ uint32_t block_base[2];
+	const uint32_t i = blockIdx.x * COMPACT_BLOCK + threadIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+	// what the blocks before this one hold
+	uint32_t a = 0, f = 0;
+	for (uint32_t k = threadIdx.x; k < blockIdx.x; k += COMPACT_BLOCK) { const U2 v = counts[k]; a += v.x; f += v.y; }
+	a = wave_sum_fast(a); f = wave_sum_fast(f);
+	const uint32_t c = compact_class(i, n, src_p, src_c);
+	const uint64_t m_alive = __ballot(c == 1u), m_fin = __ballot(c == 2u);
+	if (lane == 0) { before[0][wave] = a; before[1][wave] = f; part[0][wave] = (uint32_t)__popcll(m_alive); part[1][wave] = (uint32_t)__popcll(m_fin); }
+	__syncthreads();
+	if (threadIdx.x < 2) {
+		uint32_t sum = initial[threadIdx.x];
+		for (uint32_t k = 0; k < COMPACT_BLOCK / 64; ++k) sum += before[threadIdx.x][k];
+		block_base[threadIdx.x] = sum;
+		// the wavefronts' offsets inside the block, in place of their counts
+		uint32_t run = 0;
+		for (uint32_t k = 0; k < COMPACT_BLOCK / 64; ++k) { const uint32_t v = part[threadIdx.x][k]; part[threadIdx.x][k] = run; run += v; }
+		if (blockIdx.x == gridDim.x - 1) {
+			*(threadIdx.x == 0 ? n_alive_counter : n_final_counter) = sum + run;
+			// for a host that waits for the number of live rays: the count with the call's stamp above it, in one store to host memory
+			if (threadIdx.x == 0 && host_word) __hip_atomic_store(host_word, ((unsigned long long)stamp << 32) | (sum + run), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+		}
+	}
+	__syncthreads();
+	const uint64_t below = (1ull << lane) - 1ull;
+	if (c == 1u) {
+		const uint32_t k = block_base[0] + part[0][wave] + (uint32_t)__popcll(m_alive & below);
 		((Payload40*)dst_p)[k] = ((const Payload40*)src_p)[i];
 		*(Float4*)(dst_c + 4 * (size_t)k) = *(const Float4*)(src_c + 4 * (size_t)i);
-	} else if (fin[i]) {
-		const uint32_t k = fin_pos[i];
+	} else if (c == 2u) {
+		const uint32_t k = block_base[1] + part[1][wave] + (uint32_t)__popcll(m_fin & below);
 		((Payload40*)fin_p)[k] = ((const Payload40*)src_p)[i];
 		*(Float4*)(fin_c + 4 * (size_t)k) = *(const Float4*)(src_c + 4 * (size_t)i);
 	}
@@ -757,6 +805,32 @@ static int launch_stream(const srf_loss_args* a, const LossConst& K, ChainScratc
 		}
 	}
 #endif
+	return SRF_OK;
+}
+
+// srf_compact_rays; alive_from_zero: the live rays are numbered from 0 whatever the counter holds (the frame loop's case: it
+// would otherwise clear the counter with a launch of its own before every round)
+int compact_rays(srf_marcher* m, uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba,
+                 srf_ray_payload* dst_payloads, float* dst_rgba, srf_ray_payload* final_payloads, float* final_rgba,
+                 uint32_t* n_alive_counter, uint32_t* n_final_counter, bool alive_from_zero, hipStream_t st, unsigned long long* host_word, uint32_t stamp) {
+	SRF_REQUIRE(m, "srf_compact_rays: NULL marcher");
+	SRF_REQUIRE(n_alive_counter && n_final_counter, "srf_compact_rays: NULL counter");
+	if (n == 0) {
+		if (alive_from_zero) return fill_u32(n_alive_counter, 1, 0u, st);
+		return SRF_OK;
+	}
+	SRF_REQUIRE(src_payloads && src_rgba && dst_payloads && dst_rgba && final_payloads && final_rgba, "srf_compact_rays: NULL buffer");
+	const uint32_t blocks = div_up(n, COMPACT_BLOCK);
+	int rc = m->compact_ws.reserve(256 + (size_t)blocks * sizeof(U2));
+	if (rc != SRF_OK) return rc;
+	uint32_t* initial = (uint32_t*)m->compact_ws.ptr;
+	U2* counts = (U2*)((char*)m->compact_ws.ptr + 256);
+	hipLaunchKernelGGL(k_compact_count, dim3(blocks), dim3(COMPACT_BLOCK), 0, st, n, src_payloads, src_rgba, counts,
+	                   (const uint32_t*)n_alive_counter, (const uint32_t*)n_final_counter, initial, alive_from_zero);
+	SRF_LAUNCH_CHECK();
+	hipLaunchKernelGGL(k_compact_move, dim3(blocks), dim3(COMPACT_BLOCK), 0, st, n, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba,
+	                   (const U2*)counts, (const uint32_t*)initial, n_alive_counter, n_final_counter, host_word, stamp);
+	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }
 
@@ -1023,28 +1097,7 @@ int srf_marcher_volume_rendering(srf_marcher_t* m, const srf_sampler_t* s, const
 int srf_compact_rays(srf_marcher_t* m, uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba,
                      srf_ray_payload* dst_payloads, float* dst_rgba, srf_ray_payload* final_payloads, float* final_rgba,
                      uint32_t* n_alive_counter, uint32_t* n_final_counter, void* stream) {
-	SRF_REQUIRE(m, "srf_compact_rays: NULL marcher");
-	if (n == 0) return SRF_OK;
-	SRF_REQUIRE(src_payloads && src_rgba && dst_payloads && dst_rgba && final_payloads && final_rgba && n_alive_counter && n_final_counter,
-	            "srf_compact_rays: NULL buffer");
-	hipStream_t st = (hipStream_t)stream;
-	const size_t stride = align_up((size_t)n * 4, 256);
-	int rc = m->compact_ws.reserve(4 * stride + scan_scratch_bytes(n));
-	if (rc != SRF_OK) return rc;
-	char* w = (char*)m->compact_ws.ptr;
-	uint32_t* alive = (uint32_t*)w; uint32_t* alive_pos = (uint32_t*)(w + stride);
-	uint32_t* fin = (uint32_t*)(w + 2 * stride); uint32_t* fin_pos = (uint32_t*)(w + 3 * stride);
-	void* scan = w + 4 * stride;
-	hipLaunchKernelGGL(k_compact_flags, dim3(div_up(n, 256)), dim3(256), 0, st, n, src_payloads, src_rgba, alive, fin);
-	SRF_LAUNCH_CHECK();
-	rc = scan_exclusive_u32(alive, alive_pos, n, n_alive_counter, n_alive_counter, scan, st);
-	if (rc != SRF_OK) return rc;
-	rc = scan_exclusive_u32(fin, fin_pos, n, n_final_counter, n_final_counter, scan, st);
-	if (rc != SRF_OK) return rc;
-	hipLaunchKernelGGL(k_compact_move, dim3(div_up(n, 256)), dim3(256), 0, st, n, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba,
-	                   (const uint32_t*)alive, (const uint32_t*)alive_pos, (const uint32_t*)fin, (const uint32_t*)fin_pos);
-	SRF_LAUNCH_CHECK();
-	return SRF_OK;
+	return srf::compact_rays(m, n, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba, n_alive_counter, n_final_counter, false, (hipStream_t)stream, nullptr, 0u);
 }
 
 int srf_shade(uint32_t n_rays, const float* rgba, const srf_ray_payload* payloads, float* frame_buffer,

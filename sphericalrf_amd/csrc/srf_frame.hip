@@ -44,7 +44,13 @@ int srf_render_frame(srf_sampler_t* s, srf_marcher_t* m, const srf_frame_args* a
 	const size_t net_bytes = align_up((size_t)n_pixels * MAX_STEPS * a->padded_output_width * (a->network_output_dtype == SRF_DTYPE_F16 ? 2 : 4), 256);
 	int rc = m->frame_ws.reserve(3 * pay_bytes + 3 * col_bytes + coord_bytes + net_bytes + 256);
 	if (rc != SRF_OK) return rc;
-	if (!m->frame_counter_host) SRF_HIP(hipHostMalloc((void**)&m->frame_counter_host, 64, hipHostMallocDefault));
+	if (!m->frame_counter_host) {
+		SRF_HIP(hipHostMalloc((void**)&m->frame_counter_host, 64, hipHostMallocMapped));
+		void* dev = nullptr;
+		if (hipHostGetDevicePointer(&dev, m->frame_counter_host, 0) == hipSuccess) m->frame_word_dev = (unsigned long long*)((char*)dev + 8);
+		else (void)hipGetLastError();
+		*(volatile unsigned long long*)(m->frame_counter_host + 2) = 0ull;
+	}
 	char* w = (char*)m->frame_ws.ptr;
 	srf_ray_payload* pay[2] = {(srf_ray_payload*)w, (srf_ray_payload*)(w + pay_bytes)};
 	srf_ray_payload* hit_pay = (srf_ray_payload*)(w + 2 * pay_bytes);
@@ -72,13 +78,31 @@ int srf_render_frame(srf_sampler_t* s, srf_marcher_t* m, const srf_frame_args* a
 	while (offset < MARCH_ITER) {       // testbed.cu:526-597
 		const uint32_t prev = dbi % 2, cur = (dbi + 1) % 2;
 		++dbi;
-		SRF_HIP(hipMemsetAsync(counters, 0, 4, st));
-		rc = srf_compact_rays(m, n_alive, pay[prev], col[prev], pay[cur], col[cur], hit_pay, hit_col, counters, counters + 1, st);
+		const uint32_t stamp = ++m->frame_stamp;
+		rc = compact_rays(m, n_alive, pay[prev], col[prev], pay[cur], col[cur], hit_pay, hit_col, counters, counters + 1, true, st, m->frame_word_dev, stamp);
 		if (rc != SRF_OK) return rc;
-		// the host decides the size of the next round, as the reference does (:540-541)
-		SRF_HIP(hipMemcpyAsync(m->frame_counter_host, counters, 4, hipMemcpyDeviceToHost, st));
-		SRF_HIP(hipStreamSynchronize(st));
-		n_alive = *m->frame_counter_host;
+		// the host decides the size of the next round, as the reference does (:540-541).  The compaction's last block stores the
+		// count, stamped with this call's number, straight into host memory; the host watches that word instead of queueing a copy
+		// and waiting for the stream to drain.  Should the word not arrive although the stream has run dry, the copy does it.
+		bool seen = false;
+		if (m->frame_word_dev) {
+			const volatile unsigned long long* word = (const volatile unsigned long long*)(m->frame_counter_host + 2);
+			for (uint32_t spins = 1; !seen; ++spins) {
+				const unsigned long long v = *word;
+				if ((uint32_t)(v >> 32) == stamp) { n_alive = (uint32_t)v; seen = true; break; }
+				if ((spins & 0xfffu) == 0u && hipStreamQuery(st) != hipErrorNotReady) {
+					const unsigned long long v2 = *word;
+					if ((uint32_t)(v2 >> 32) == stamp) { n_alive = (uint32_t)v2; seen = true; }
+					break;
+				}
+			}
+			(void)hipGetLastError();
+		}
+		if (!seen) {
+			SRF_HIP(hipMemcpyAsync(m->frame_counter_host, counters, 4, hipMemcpyDeviceToHost, st));
+			SRF_HIP(hipStreamSynchronize(st));
+			n_alive = *m->frame_counter_host;
+		}
 		if (n_alive == 0) break;
 		++iters;
 		uint32_t n_steps = n_pixels / n_alive;

@@ -68,9 +68,11 @@ struct srf_marcher {
 	srf::Workspace ws;          // ordered-offset chain of the streaming compositing kernel
 	srf::Workspace ws2;         // per-ray forward results of the three-launch compositing
 	srf::Workspace reg;         // reg_distortion_buffer (ray_marcher.h:79-80)
-	srf::Workspace compact_ws;  // flags and positions of srf_marcher_compact_rays
+	srf::Workspace compact_ws;  // per-block counts of srf_compact_rays
 	srf::Workspace frame_ws;    // ray buffers, coordinates and network output of srf_render_frame
-	uint32_t* frame_counter_host = nullptr;  // pinned word through which srf_render_frame reads the ray counters
+	uint32_t* frame_counter_host = nullptr;  // pinned words through which srf_render_frame reads the ray counters
+	unsigned long long* frame_word_dev = nullptr;   // device address of the second of them (8 bytes in), which the compaction kernel writes itself
+	uint32_t frame_stamp = 0;                // number of the last compaction srf_render_frame waited for
 	bool force_unfused = false;             // SRF_COMPOSITE_IMPL=unfused at creation
 	bool degraded = false;                  // the chain has failed once: every later call uses the three-launch implementation
 	volatile uint32_t* host_error = nullptr; // host word the streaming kernel raises when its chain gives up (pinned, device-writable)
@@ -78,3 +80,12 @@ struct srf_marcher {
 	uint32_t* chain_error_dev = nullptr;     // device word of the last streaming launch (NULL before the first)
 	uint32_t lookback_spin_limit = 1u << 22; // polls before a group gives up waiting for its predecessors
 };
+
+namespace srf {
+// srf_compact_rays with two more choices: alive_from_zero numbers the live rays from 0 whatever *n_alive_counter holds; host_word
+// (device address of a word of host memory, or NULL) receives stamp << 32 | the live-ray counter's new value when the call is done
+int compact_rays(srf_marcher* m, uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba,
+                 srf_ray_payload* dst_payloads, float* dst_rgba, srf_ray_payload* final_payloads, float* final_rgba,
+                 uint32_t* n_alive_counter, uint32_t* n_final_counter, bool alive_from_zero, hipStream_t stream,
+                 unsigned long long* host_word, uint32_t stamp);
+}
