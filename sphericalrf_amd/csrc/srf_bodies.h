@@ -545,18 +545,19 @@ SRF_HD uint64_t low_bits64(uint32_t n) { return n >= 64u ? ~0ull : (1ull << n) -
 SRF_HD uint64_t wide_chain(const Params& P, float t0, float* t) {
 	const ShortForm f = disparity_short_form(P);
 	if (f.usable && t0 >= f.t_lo) {
-		// the whole batch in the short form, checked afterwards: t only grows, so the last step's start bounds them all,
-		// and inside the short form's range every step is positive
+		// the whole batch in the short form, checked afterwards; inside the short form's range every step is positive
 		ShortChain ch = short_chain_at(t0);
+		bool in_range = true;      // past the range the chain runs through infinity to negative values: every start is looked at
 #if defined(__HIP_DEVICE_COMPILE__)
 		#pragma unroll 8
 #endif
 		for (uint32_t k = 0; k < WIDE_STEPS; ++k) {
 			t[k] = ch.t;
+			in_range = in_range & (ch.t <= f.t_hi) & (ch.t >= f.t_lo);
 			ch = short_chain_next(f, ch);
 		}
 		t[WIDE_STEPS] = ch.t;
-		if (t[WIDE_STEPS - 1] <= f.t_hi) return 0ull;
+		if (in_range) return 0ull;
 	}
 	uint64_t zero = 0;
 	float tk = t0;
@@ -839,11 +840,14 @@ SRF_HD void init_ray_body(uint32_t x, uint32_t y, const Params& P, const PixelAr
 // goes on.  A wavefront runs its lanes' phases by majority (srf_march.hip); one lane alone runs them in turn.
 // ------------------------------------------------------------------------------------
 enum MarchEnd : uint32_t { MARCH_GOES_ON = 0, MARCH_LEFT_BOX = 1, MARCH_ZERO_STEP = 2, MARCH_STOPPED = 3, MARCH_NO_RAY = 4 };
-struct MarchLane { uint32_t phase; Vec3 o, d; float t, t_limit; SkipRay sr; };
+// crawl: how many probes in a row found an empty cell and nothing to skip (the ray runs through occupied surroundings and looks a
+// cell up at every step); the last few rays of a wavefront that crawl are handed to the one-ray-per-wavefront march (srf_march.hip)
+struct MarchLane { uint32_t phase, crawl; Vec3 o, d; float t, t_limit; SkipRay sr; };
 
 SRF_HD void march_start(MarchLane& L, Vec3 o, Vec3 d, float t, bool skipping) {
 	L.o = o; L.d = d;
 	L.t = L.t_limit = t;
+	L.crawl = 0;
 	if (skipping) L.sr = skip_ray_setup(o, d);
 	L.phase = LANE_PROBE;
 }
@@ -869,11 +873,14 @@ SRF_HD MarchEnd march_probe(MarchLane& L, const Params& P, const uint8_t* bitfie
 	SRF_COUNT_PROBE();
 	const Probe s = probe_at(P, bitfield, pos, L.t, cone, &skip);
 	L.t_limit = L.t;      // steps at t' < t_limit are known to find an empty cell
+	const uint32_t crawled = L.crawl;
+	L.crawl = 0;
 	if (s.occ) return hit(L, s);
 	if (skipping) L.t_limit = skip_limit(P, skip, L.sr, L.o, L.d, L.t, s.radius, s.level);
 	L.t += s.dt;
 	if (s.dt == 0.f) return MARCH_ZERO_STEP;
 	L.phase = L.t < L.t_limit ? LANE_STEP : LANE_PROBE;
+	L.crawl = L.phase == LANE_PROBE ? crawled + 1u : 0u;
 	return MARCH_GOES_ON;
 }
 

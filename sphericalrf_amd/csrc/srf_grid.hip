@@ -423,6 +423,9 @@ int srf_sampler_create(const srf_sampler_config* c, srf_sampler_t** out) {
 	s->force_sample_by_cell = tri_state("SRF_GRID_SAMPLE_BY_CELL");
 	s->count_probe_budget = COUNT_PROBE_BUDGET;
 	{ const char* v = getenv("SRF_COUNT_PROBE_BUDGET"); if (v && v[0]) s->count_probe_budget = (uint32_t)atoi(v); }
+	// SRF_MARCH_PARK_ALL=1: the render marches hand every ray that finds an empty cell without anything to skip to their
+	// one-ray-per-wavefront march at once, whatever the wavefront still holds (for tests: that march then does most of a frame)
+	{ const char* v = getenv("SRF_MARCH_PARK_ALL"); s->march_park_all = v && v[0] == '1'; }
 	hipError_t e = hipSuccess;
 	if (P.use_grid) {
 		e = hipMalloc((void**)&s->density_grid_current, (size_t)s->n_total * sizeof(float));
@@ -452,6 +455,8 @@ void srf_sampler_destroy(srf_sampler_t* s) {
 	if (s->density_grid_bitfield) (void)hipFree(s->density_grid_bitfield);
 	if (s->skip_dist) (void)hipFree(s->skip_dist);
 	s->ws.release();
+	s->park_ws.release();
+	if (s->park_counts) (void)hipFree(s->park_counts);
 	delete s;
 }
 

@@ -61,6 +61,10 @@ struct srf_sampler {
 	int      force_splat_sort, force_sample_bits, force_sample_by_cell;
 	uint32_t count_probe_budget;
 	srf::Workspace ws;
+	srf::Workspace park_ws;          // queue of the rays the render marches hand to their one-ray-per-wavefront march
+	uint32_t* park_counts = nullptr; // two counters of that queue, used in turn: a march clears the one the next march will use
+	uint32_t park_turn = 0;
+	bool march_park_all = false;     // SRF_MARCH_PARK_ALL at creation
 };
 
 struct srf_marcher {

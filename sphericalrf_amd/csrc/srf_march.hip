@@ -4,6 +4,7 @@
 #include <stdlib.h>
 #include "srf_internal.h"
 #include "srf_bodies.h"
+#include "srf_wave.h"
 
 namespace srf {
 
@@ -241,12 +242,98 @@ __global__ void __launch_bounds__(128) k_init_rays(Params P, PixelArgs A, srf_ra
 // Letting the probing lanes go first once they outnumber the stepping ones, and stepping in bursts of a fixed length (as the
 // counting march does), costs 5 to 15 % of a frame on the render workloads: here most lanes walk the same long empty
 // stretches side by side.
+// A ray that crawls (an empty cell and nothing to skip at every probe: it runs along occupied blocks) costs a round of dependent
+// loads a step, and when it is one of the last few rays of its wavefront nothing hides them: such rays alone kept a frame of the
+// bounded-object workload alive four times longer than its average wavefront.  A wavefront down to PARK_MAX_LANES rays therefore
+// parks those that have crawled PARK_CRAWL probes in a row: the lane's state goes to a queue as it stands, and k_march_wide
+// carries each parked ray on, one ray a wavefront.  There a crawling ray is taken through its next 64 steps at once: every lane
+// follows the chain of t (it has to be followed step by step) and keeps the value before its own step, looks that position up, and
+// the first step that is not "inside, empty, of positive size" is where the ray's own probe carries on; nothing else of the
+// ray's state moves, so the march's outcome is the one of probing step by step.
+// (settled on the render workloads: parking after 16 or 32 probes costs the frames without such rays 5 to 10 % in rays that
+// would have stopped crawling soon; wide rounds inside the march kernel itself cost them more than that in registers)
+constexpr uint32_t PARK_MAX_LANES = 8, PARK_CRAWL = 64;
+struct MarchPark { void* slots; uint32_t* count; uint32_t* next_count; uint32_t capacity, max_lanes, min_crawl; };
+
+__device__ __forceinline__ float lane_value_f32(float v, uint32_t uniform_lane) { return srf_u2f(lane_value_u32(srf_f2u(v), uniform_lane)); }
+// the ray in lane `owner`; true when the next 64 steps held nothing (the ray may go wide again at once)
+__device__ inline bool march_wide_round(const MarchGrid& G, MarchLane& L, uint32_t owner) {
+	const Params& P = G.P;
+	const uint32_t lane = threadIdx.x & 63u;
+	const float cone = P.cone_angle_constant;
+	const Vec3 o = mk3(lane_value_f32(L.o.x, owner), lane_value_f32(L.o.y, owner), lane_value_f32(L.o.z, owner));
+	const Vec3 d = mk3(lane_value_f32(L.d.x, owner), lane_value_f32(L.d.y, owner), lane_value_f32(L.d.z, owner));
+	const float t0 = lane_value_f32(L.t, owner);
+	float t_mine = t0, t_end = t0;
+	bool zero_mine = false, chained = false;
+	const ShortForm f = disparity_short_form(P);
+	if (f.usable && t0 >= f.t_lo) {
+		// the whole batch in the short form, checked afterwards: every step must start inside the form's range (past it the chain
+		// runs through infinity to negative values, so the last step's start alone does not tell)
+		ShortChain ch = short_chain_at(t0);
+		for (uint32_t k = 0; k < 64u; ++k) {
+			t_mine = k == lane ? ch.t : t_mine;
+			ch = short_chain_next(f, ch);
+		}
+		t_end = ch.t;
+		chained = __ballot(!(t_mine >= f.t_lo && t_mine <= f.t_hi)) == 0ull;
+	}
+	if (!chained) {
+		float t = t0;
+		for (uint32_t k = 0; k < 64u; ++k) {
+			const float dt = calc_dt(P, t, cone);
+			if (k == lane) { t_mine = t; zero_mine = dt == 0.f; }
+			t += dt;
+		}
+		t_end = t;
+	}
+	const Vec3 pos = along(o, d, t_mine);
+	bool event = !aabb_contains(P, pos) || zero_mine;
+	if (!event) {
+		bool look = true;
+		if (P.sphere[3] > 0.f) {
+			float t_enter;
+			const SphereGate g = sphere_gate(P, o, d, t_mine, &t_enter);
+			event = g == SPHERE_BEYOND;
+			look = g == SPHERE_INSIDE;
+		}
+		if (look) event = probe_at(P, G.bitfield, pos, t_mine, cone).occ;
+	}
+	const uint64_t m = __ballot(event);
+	const float t_new = m ? lane_value_f32(t_mine, (uint32_t)__builtin_ctzll(m)) : t_end;
+	if (lane == owner) { L.t = L.t_limit = t_new; L.phase = LANE_PROBE; if (m) L.crawl = 0; }
+	return m == 0ull;
+}
+
+// the parked rays, one a wavefront: lane 0 carries the ray's state and runs its probes and steps, all lanes its wide rounds
+template <class March>
+__global__ void __launch_bounds__(64) k_march_wide(March M, MarchPark park) {
+	const uint32_t lane = threadIdx.x;
+	const uint32_t filled = *park.count;
+	const uint32_t n = filled < park.capacity ? filled : park.capacity;
+	for (uint32_t q = blockIdx.x; q < n; q += gridDim.x) {
+		typename March::Lane L;
+		L.m.phase = LANE_IDLE; L.m.crawl = 0;
+		L.m.o = mk3(0.f, 0.f, 0.f); L.m.d = L.m.o; L.m.t = 0.f;
+		if (lane == 0) L = ((const typename March::Lane*)park.slots)[q];
+		for (;;) {
+			const uint32_t phase = lane_value_u32(L.m.phase, 0u);
+			if (phase == LANE_IDLE) break;
+			MarchEnd end = MARCH_GOES_ON;
+			if (phase == LANE_STEP) { if (lane == 0) end = M.steps(L); }
+			else if (lane_value_u32(L.m.crawl, 0u) != 0u) march_wide_round(M.G, L.m, 0u);
+			else if (lane == 0) end = M.probe(L);
+			if (lane == 0 && end != MARCH_GOES_ON) { M.finish(L, end); L.m.phase = LANE_IDLE; }
+		}
+	}
+}
+
 #ifdef SRF_KERNEL_TIMING
 // per phase (step, probe): cycles, rounds, lanes that took part; then wavefronts, their lifetime in cycles, the longest in 10 ns ticks
 __device__ unsigned long long g_march_timing[16];
 #endif
 template <class March>
-__global__ void __launch_bounds__(64) k_march_lanes(March M) {
+__global__ void __launch_bounds__(64) k_march_lanes(March M, MarchPark park) {
 	const uint32_t q = blockIdx.x * 64u + threadIdx.x;
 	typename March::Lane L;
 	L.m.phase = LANE_IDLE;
@@ -258,6 +345,7 @@ __global__ void __launch_bounds__(64) k_march_lanes(March M) {
 #else
 #define SRF_MARCH_STAMP(k, lanes) ((void)0)
 #endif
+	if (q == 0 && park.next_count) *park.next_count = 0u;      // the queue counter of the march after this one
 	// a lane's march ends in begin, probe or steps; its results are stored in one place, here
 	MarchEnd end = q < M.lanes() ? M.begin(L, q) : MARCH_NO_RAY;
 	for (;;) {
@@ -274,6 +362,12 @@ __global__ void __launch_bounds__(64) k_march_lanes(March M) {
 			SRF_MARCH_STAMP(0, n_step);
 		} else {
 			if (L.m.phase == LANE_PROBE) end = M.probe(L);
+			// one of the wavefront's last few rays, crawling: it carries on in k_march_wide
+			if (n_probe <= park.max_lanes && end == MARCH_GOES_ON && L.m.phase == LANE_PROBE && L.m.crawl >= park.min_crawl) {
+				const uint32_t slot = atomicAdd(park.count, 1u);
+				if (slot < park.capacity) { ((typename March::Lane*)park.slots)[slot] = L; L.m.phase = LANE_IDLE; }
+				else L.m.crawl = 0;      // the queue is full: the ray stays
+			}
 			SRF_MARCH_STAMP(1, n_probe);
 		}
 	}
@@ -287,12 +381,29 @@ __global__ void __launch_bounds__(64) k_march_lanes(March M) {
 #endif
 }
 
+// the march and, behind it, the wide march of the rays it parked
 template <class March>
-static void launch_march(const March& M, hipStream_t st) {
-	hipLaunchKernelGGL(k_march_lanes<March>, dim3(div_up(M.lanes(), 64u)), dim3(64), 0, st, M);
+static int launch_march(const March& M, srf_sampler* s, hipStream_t st) {
+	const uint32_t n = M.lanes();
+	MarchPark park;
+	park.capacity = s->march_park_all ? n : n / 8u + 64u;
+	park.max_lanes = s->march_park_all ? 64u : PARK_MAX_LANES;
+	park.min_crawl = s->march_park_all ? 1u : PARK_CRAWL;
+	int rc = s->park_ws.reserve((size_t)park.capacity * sizeof(typename March::Lane));
+	if (rc != SRF_OK) return rc;
+	if (!s->park_counts) {
+		SRF_HIP(hipMalloc((void**)&s->park_counts, 256));
+		SRF_HIP(hipMemset(s->park_counts, 0, 256));
+	}
+	park.slots = s->park_ws.ptr;
+	park.count = s->park_counts + (s->park_turn & 1u);
+	park.next_count = s->park_counts + ((s->park_turn + 1u) & 1u);
+	++s->park_turn;
+	hipLaunchKernelGGL(k_march_lanes<March>, dim3(div_up(n, 64u)), dim3(64), 0, st, M, park);
+	hipLaunchKernelGGL(k_march_wide<March>, dim3(park.capacity < 4096u ? park.capacity : 4096u), dim3(64), 0, st, M, park);
 #ifdef SRF_KERNEL_TIMING
 	unsigned long long h[16], zero[16] = {0};
-	if (hipStreamSynchronize(st) != hipSuccess || hipMemcpyFromSymbol(h, HIP_SYMBOL(g_march_timing), sizeof(h)) != hipSuccess) return;
+	if (hipStreamSynchronize(st) != hipSuccess || hipMemcpyFromSymbol(h, HIP_SYMBOL(g_march_timing), sizeof(h)) != hipSuccess) return SRF_OK;
 	(void)hipMemcpyToSymbol(HIP_SYMBOL(g_march_timing), zero, sizeof(zero));
 	const double nw = (double)(h[6] ? h[6] : 1);
 	fprintf(stderr, "march of %u lanes: wavefront lifetime %.0f cycles mean, %.1f us longest\n", M.lanes(), (double)h[7] / nw, (double)h[8] / 100.0);
@@ -300,7 +411,10 @@ static void launch_march(const March& M, hipStream_t st) {
 	for (int k = 0; k < 2; ++k)
 		fprintf(stderr, "march %-5s: %.0f cycles per wavefront, %.1f rounds, %.0f cycles per round, %.1f lanes per round\n", name[k],
 		        (double)h[k] / nw, (double)h[2 + k] / nw, h[2 + k] ? (double)h[k] / (double)h[2 + k] : 0.0, h[2 + k] ? (double)h[4 + k] / (double)h[2 + k] : 0.0);
+	{ uint32_t n_parked = 0; if (hipMemcpy(&n_parked, park.count, 4, hipMemcpyDeviceToHost) == hipSuccess) fprintf(stderr, "march parked %u rays (capacity %u)\n", n_parked, park.capacity); }
 #endif
+	SRF_LAUNCH_CHECK();
+	return SRF_OK;
 }
 
 // the stretch of every ray inside a sphere; a ray that misses it gets the empty stretch (+inf, -inf).  24 B in, 8 B out a ray.
@@ -519,9 +633,7 @@ int srf_sampler_generate_rays_from_camera_matrix(srf_sampler_t* s, const int32_t
 	const uint32_t n = (uint32_t)resolution[0] * (uint32_t)resolution[1];
 	AdvanceMarch M;
 	M.G = sampler_march_grid(s); M.n_rays = n; M.spp = spp; M.payloads = payload;
-	launch_march(M, st);
-	SRF_LAUNCH_CHECK();
-	return SRF_OK;
+	return launch_march(M, s, st);
 }
 
 int srf_sampler_generate_coords_from_rays(srf_sampler_t* s, uint32_t n_rays, uint32_t n_steps,
@@ -531,9 +643,7 @@ int srf_sampler_generate_coords_from_rays(srf_sampler_t* s, uint32_t n_rays, uin
 	SRF_REQUIRE(payloads && coords, "srf_sampler_generate_coords_from_rays: NULL buffer");
 	CoordsMarch M;
 	M.G = sampler_march_grid(s); M.n_rays = n_rays; M.n_steps = n_steps; M.payloads = payloads; M.coords = coords;
-	launch_march(M, (hipStream_t)stream);
-	SRF_LAUNCH_CHECK();
-	return SRF_OK;
+	return launch_march(M, s, (hipStream_t)stream);
 }
 
 int srf_field_eval(const srf_sampler_t* s, const srf_field* field, uint32_t n_coords, const float* coords,
@@ -569,9 +679,7 @@ int srf_render_frame_fused(srf_sampler_t* s, const srf_marcher_t* m, const srf_f
 	M.F.table = field->table; M.F.mask = field->table_size - 1; M.F.seed = field->seed;
 	M.thr = m->cfg.transmittance_threshold; M.to_linear = m->cfg.train_in_linear_color ? 0 : 1;
 	M.frame = frame_buffer; M.n_samples = n_samples;
-	launch_march(M, (hipStream_t)stream);
-	SRF_LAUNCH_CHECK();
-	return SRF_OK;
+	return launch_march(M, s, (hipStream_t)stream);
 }
 
 } // extern "C"

@@ -1,7 +1,9 @@
 // Torch-free driver of one training step (march + compositing forward/backward) through include/srf_hip.hpp,
 // for timing and for profiler runs (a process that holds nothing but this library's kernels and a few fill kernels).
 //
-//   step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite] [--verify] [--copy-check]
+//   step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite|render] [--verify] [--copy-check]
+//
+// --only render times whole frames of the workload file's cameras through srf_render_frame_fused instead (any workload).
 //
 // The workload file (written by sphericalrf_amd.scene.write_workload_file) holds the sampler configuration, the
 // cameras, the occupancy bitfield and a table of (r, g, b, sigma) rows; per-sample network output and per-ray targets
@@ -102,7 +104,7 @@ struct Timer {
 };
 
 int main(int argc, char** argv) {
-	if (argc < 2) { std::fprintf(stderr, "usage: step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite] [--verify] [--copy-check]\n"); return 2; }
+	if (argc < 2) { std::fprintf(stderr, "usage: step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite|render] [--verify] [--copy-check]\n"); return 2; }
 	uint32_t steps = 10, warmup = 2, n_rays = 1u << 20, cap = 1u << 24;
 	bool verify = false, copy_check = false;
 	std::string only;
@@ -146,6 +148,32 @@ int main(int argc, char** argv) {
 		mc.train_in_linear_color = 1;
 		mc.transmittance_threshold = 1e-4f;
 		srf::RayMarcher marcher(mc);
+
+		if (only == "render") {
+			// frames of the workload's cameras in turn through the one-launch frame, the table standing in for the network
+			const uint32_t n_pixels = (uint32_t)w.res[0] * (uint32_t)w.res[1];
+			float* frame = dev_alloc<float>((size_t)n_pixels * 4);
+			uint32_t* n_samples = dev_alloc<uint32_t>(n_pixels);
+			float* d_table = dev_alloc<float>(w.table.size());
+			HIP_OK(hipMemcpy(d_table, w.table.data(), w.table.size() * 4, hipMemcpyHostToDevice));
+			srf_field field{d_table, (uint32_t)(w.table.size() / 4), 1000u};
+			const float pp[2] = {0.5f, 0.5f};
+			Timer tm;
+			double ms = 0;
+			for (uint32_t k = 0; k < warmup + steps; ++k) {
+				tm.start(st);
+				const int rc = srf_render_frame_fused(sampler.handle(), marcher.handle(), &field, w.res, w.focal, pp, &w.cameras[(size_t)(k % w.n_cameras) * 12], 0, frame, n_samples, st);
+				if (rc != SRF_OK) { std::fprintf(stderr, "srf_render_frame_fused: %s\n", srf_last_error()); return 1; }
+				const float t = tm.stop(st);
+				if (k >= warmup) ms += t;
+			}
+			std::vector<uint32_t> ns(n_pixels);
+			HIP_OK(hipMemcpy(ns.data(), n_samples, (size_t)n_pixels * 4, hipMemcpyDeviceToHost));
+			unsigned long long total = 0;
+			for (uint32_t v : ns) total += v;
+			std::printf("{\"frames\": %u, \"resolution\": [%d, %d], \"render_ms\": %.4f, \"composited_samples_last_frame\": %llu}\n", steps, w.res[0], w.res[1], ms / steps, total);
+			return 0;
+		}
 
 		float* d_cams = dev_alloc<float>(w.cameras.size());
 		HIP_OK(hipMemcpy(d_cams, w.cameras.data(), w.cameras.size() * 4, hipMemcpyHostToDevice));

@@ -484,6 +484,38 @@ def test_every_loss_function(gpu, orc, loss, impl, monkeypatch):
     assert np.abs(o_dloss).max() > 0
 
 
+@pytest.mark.parametrize("config_id,scale", [(1, 0.5), (2, 0.25), (3, 0.125)])
+def test_render_marches_through_the_one_ray_per_wavefront_march(gpu, orc, config_id, scale, monkeypatch):
+    """SRF_MARCH_PARK_ALL=1 sends every ray that looks a cell up at every step to the march that takes one ray a wavefront through 64
+    steps at once (in a normal run only the last few rays of a wavefront go there, after 64 such steps): fused frame, first hits
+    and two rounds of coordinates against the oracle"""
+    torch = gpu
+    monkeypatch.setenv("SRF_MARCH_PARK_ALL", "1")
+    from sphericalrf_amd import api, scene
+    w, p, grid, bf, mean = helpers.build_scene(orc, config_id, scale)
+    s = make_sampler(torch, api, w, grid)
+    monkeypatch.delenv("SRF_MARCH_PARK_ALL")
+    m = api.RayMarcher(dict(train_in_linear_color=False, transmittance_threshold=1e-4))
+    res, f, cam = w["resolution"], w["focal"], w["cameras"][-1]
+    n = res[0] * res[1]
+    table = scene.field_table(4096, 5)
+    table[:, 3] *= 20
+    want_frame, want_ns, _ = orc.render_frame(p, orc.make_field(table, 77), bf, res, f, (0.5, 0.5), cam, transmittance_threshold=1e-4, train_in_linear_colors=False)
+    frame, ns = torch.ones((res[1], res[0], 4), device="cuda"), torch.zeros(n, dtype=torch.int32, device="cuda")
+    s.render_frame_fused(m, api.Field(torch.from_numpy(table).cuda(), 77), res, f, (0.5, 0.5), cam, frame, ns)
+    assert np.array_equal(u32(ns).reshape(res[1], res[0]), want_ns) and np.array_equal(frame.cpu().numpy(), want_frame)
+    pay = torch.zeros(n * 40, dtype=torch.uint8, device="cuda")
+    s.generate_rays_from_camera_matrix(res, f, (0.5, 0.5), cam, pay)
+    o_pay = orc.init_rays_with_payload(p, res, f, (0.5, 0.5), cam)
+    orc.advance_pos(p, o_pay, bf)
+    assert np.array_equal(pay.cpu().numpy().view(O.PAYLOAD_DTYPE), o_pay) and (o_pay["alive"] == 1).mean() > 0.05
+    for n_steps in (3, 8):
+        g_coords, o_coords = torch.zeros((n * n_steps, 7), device="cuda"), np.zeros((n * n_steps, 7), np.float32)
+        s.generate_coords_from_rays(n, n_steps, pay, g_coords)
+        orc.generate_coords_from_rays(p, n, n_steps, bf, o_pay, o_coords)
+        assert np.array_equal(pay.cpu().numpy().view(O.PAYLOAD_DTYPE), o_pay) and np.array_equal(g_coords.cpu().numpy(), o_coords)
+
+
 @pytest.mark.parametrize("res", [(37, 21), (8, 8), (9, 70), (131, 5), (1, 1)])
 def test_fused_frame_sizes_that_do_not_fill_their_pixel_tiles(gpu, orc, res):
     """the fused frame hands 8 x 8 pixel tiles to its wavefronts: widths and heights that leave tiles partly outside the frame"""
