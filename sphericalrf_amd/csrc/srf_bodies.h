@@ -547,17 +547,17 @@ SRF_HD uint64_t wide_chain(const Params& P, float t0, float* t) {
 	if (f.usable && t0 >= f.t_lo) {
 		// the whole batch in the short form, checked afterwards; inside the short form's range every step is positive
 		ShortChain ch = short_chain_at(t0);
-		bool in_range = true;      // past the range the chain runs through infinity to negative values: every start is looked at
 #if defined(__HIP_DEVICE_COMPILE__)
 		#pragma unroll 8
 #endif
 		for (uint32_t k = 0; k < WIDE_STEPS; ++k) {
 			t[k] = ch.t;
-			in_range = in_range & (ch.t <= f.t_hi) & (ch.t >= f.t_lo);
 			ch = short_chain_next(f, ch);
 		}
 		t[WIDE_STEPS] = ch.t;
-		if (in_range) return 0ull;
+		// t grows until, past the range, the chain runs through infinity; from there on it is negative for good: a last start
+		// that is positive and inside the range says that all of them were
+		if (t[WIDE_STEPS - 1] >= f.t_lo && t[WIDE_STEPS - 1] <= f.t_hi) return 0ull;
 	}
 	uint64_t zero = 0;
 	float tk = t0;
@@ -573,12 +573,13 @@ SRF_HD uint64_t wide_chain(const Params& P, float t0, float* t) {
 
 // the lookup of one position in two halves, so that other work can run while the occupancy byte is on its way
 struct WideLookup { uint32_t byte, bit; bool inside; };
+template <bool SPHERE = true>
 SRF_HD WideLookup wide_lookup(const Params& P, const CountArgs& A, Vec3 o, Vec3 d, float t) {
 	WideLookup q;
 	const Vec3 pos = along(o, d, t);
 	q.inside = aabb_contains(P, pos);
 	q.byte = 0xffu; q.bit = 0u;
-	if (q.inside && P.sphere[3] > 0.f) {
+	if (SPHERE && q.inside && P.sphere[3] > 0.f) {
 		float t_enter;
 		const SphereGate g = sphere_gate(P, o, d, t, &t_enter);
 		if (g == SPHERE_BEYOND) q.inside = false;

@@ -116,6 +116,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(SRF_COU
 // The wide march of the parked rays: one ray per workgroup of two wavefronts at a time.  The second wavefront runs the
 // chain of t one round (64 steps) ahead, since the step sizes do not depend on what the grid holds; in the first, every
 // lane looks one of the current round's 64 positions up and lane 0 replays the loop's bookkeeping over the results.
+template <bool SPHERE>
 __global__ void __launch_bounds__(128) k_train_count_wide(Params P, CountArgs A) {
 	__shared__ float t[2][WIDE_STEPS + 1];
 	__shared__ uint64_t zero_steps[2];
@@ -134,7 +135,7 @@ __global__ void __launch_bounds__(128) k_train_count_wide(Params P, CountArgs A)
 				// the next round starts where this one ends, if the ray gets that far
 				if (lane == 0) zero_steps[cur ^ 1u] = wide_chain(P, t[cur][WIDE_STEPS], t[cur ^ 1u]);
 			} else {
-				const uint32_t f = wide_flags(wide_lookup(P, A, L.o, L.d, t[cur][lane]));
+				const uint32_t f = wide_flags(wide_lookup<SPHERE>(P, A, L.o, L.d, t[cur][lane]));
 				const uint64_t m_inside = __ballot((f & 1u) != 0u), m_occ = __ballot((f & 2u) != 0u);
 				if (lane == 0) {
 					wide_apply(L, P, A, t[cur], m_inside, m_occ, zero_steps[cur]);
@@ -583,7 +584,8 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 	SRF_LAUNCH_CHECK();
 	if (probe_budget) {
 		const uint32_t wide_blocks = parked_capacity < 4096u ? parked_capacity : 4096u;
-		hipLaunchKernelGGL(k_train_count_wide, dim3(wide_blocks), dim3(128), 0, st, s->P, ca);
+		if (s->P.sphere[3] > 0.f) hipLaunchKernelGGL(k_train_count_wide<true>, dim3(wide_blocks), dim3(128), 0, st, s->P, ca);
+		else hipLaunchKernelGGL(k_train_count_wide<false>, dim3(wide_blocks), dim3(128), 0, st, s->P, ca);
 		SRF_LAUNCH_CHECK();
 	}
 	rc = scan_exclusive_u32(counts, base, n_rays, n_coords_counter, n_coords_counter, scan, st);
