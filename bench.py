@@ -204,10 +204,20 @@ def bench_render(torch, api, scene, config_id, steps, warmup, n_frames=2):
 
     sec = timed(torch, step, steps, warmup)
     total = int(ns.long().sum().item())
+    # the same frames through the reference's loop of entry points run inside the library (srf_render_frame), the table as the network
+    rounds = {"n": 0}
+
+    def loop_step():
+        rounds["n"] = s.render_frame(m, field, res, w["focal"], (0.5, 0.5), cams[k["i"] % len(cams)], frame, density_activation=api.ACT_NONE,
+                                     rgb_activation=api.ACT_NONE, network_output_dtype=api.DTYPE_F32)
+        k["i"] += 1
+
+    k["i"] = 0
+    loop_sec = timed(torch, loop_step, steps, warmup)
     bits = s.density_grid_bitfield
     occ = float(torch.from_numpy(__import__("numpy").unpackbits(bits.cpu().numpy())).float().mean())
     return dict(workload="render_%d" % config_id, resolution=list(res), ms_per_frame=sec * 1e3, rays_per_s=n / sec, composited_samples_last_frame=total,
-                samples_per_s=total / sec, occupied_bits=occ, frames_in_workload=len(cams))
+                samples_per_s=total / sec, loop_ms_per_frame=loop_sec * 1e3, loop_rounds_last_frame=rounds["n"], occupied_bits=occ, frames_in_workload=len(cams))
 
 
 def bench_grid_update(torch, api, scene, steps, warmup):
