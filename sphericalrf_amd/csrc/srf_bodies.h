@@ -888,13 +888,47 @@ SRF_HD MarchEnd march_probe(MarchLane& L, const Params& P, const uint8_t* bitfie
 // the steps below t_limit, each lane for itself; the step sizes are count_steps's (the short form of the disparity chain
 // where it holds, calc_dt elsewhere), and a step of size zero ends the march.  The plain loop that lanes leave one by one
 // (seven vector instructions a step) beats predicated bursts of a fixed length here, where all lanes step before any probes.
+//
+// Half of the way the chain is plainer still.  For a float g whose mantissa is below sqrt 2, the reciprocal of its reciprocal
+// (both correctly rounded) is g itself: RN(1/g) is off by at most half an ulp of a number with mantissa 2/m, which moves its
+// reciprocal by less than half an ulp of g when m^2 < 2 (every such mantissa checked: tests/test_disparity_chain.py).  While
+// g = c + 1/t stays in that lower part [2^e, sqrt 2 * 2^e) of one binade, the reciprocal the chain carries is therefore g, a
+// step is one addition, and t = RN(1/g) is only needed when the stretch ends.  "t < lim" becomes "r > G" with a margin of
+// 2^-21 (r > G implies RN(1/r) < lim; what the margin leaves is taken by the chained form, which gives the same values).  As
+// g falls, the upper part of a binade (chained steps) and its lower part (additions) take turns, a few hundred steps each.
+constexpr uint32_t MARCH_PLAIN_MIN_STEPS = 24;
 SRF_HD MarchEnd march_steps(MarchLane& L, const Params& P) {
 	const float cone = P.cone_angle_constant;
 	const ShortForm f = disparity_short_form(P);
 	if (f.usable && L.t >= f.t_lo) {
 		const float lim = srf_min(L.t_limit, f.t_hi);
 		ShortChain ch = short_chain_at(L.t);
-		while (ch.t < lim) ch = short_chain_next(f, ch);
+		const float G = srf_approx_rcp(lim) * 1.000001f;      // 1 + 2^-20: the estimate's ulp, the product's rounding and an ulp between t and RN(1/r)
+		// a stretch of a few steps is not worth telling the two forms apart: (r - G) / -c estimates its length
+		if (!(ch.r - G > -(float)MARCH_PLAIN_MIN_STEPS * f.c)) {
+			while (ch.t < lim) ch = short_chain_next(f, ch);
+		} else if (ch.t < lim) {
+			do {
+				const float g1 = f.c + ch.r;
+				const float bin = srf_u2f(srf_f2u(g1) & 0x7f800000u);      // 2^e <= g1
+				if (g1 > 0.f && g1 < bin * 1.4142134f) {
+					// additions while the step still lands at or above 2^e (r > 2^e - c, rounded up) and t is still below lim
+					const float S = srf_max(G, (bin - f.c) * 1.0000002f);
+					float r = ch.r;
+					if (r > S) {
+						do r = f.c + r; while (r > S);
+						ch.r = r;
+						ch.t = srf_rcp_normal(r);
+					} else {
+						ch = short_chain_next(f, ch);      // at the end of the stretch or of the binade's lower part
+					}
+				} else {
+					// chained steps up to where g enters the lower part of its binade: g < sqrt 2 * 2^e, t > 1 / (sqrt 2 * 2^e)
+					const float lim_c = srf_min(lim, srf_approx_rcp(bin * 1.4142134f) * 1.000001f);
+					do ch = short_chain_next(f, ch); while (ch.t < lim_c);
+				}
+			} while (ch.t < lim);
+		}
 		L.t = ch.t;
 	}
 	while (L.t < L.t_limit) {      // what the short form does not cover
