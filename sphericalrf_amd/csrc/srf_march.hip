@@ -18,9 +18,8 @@ namespace srf {
 // 16: 1.91 ms, 24: 1.66 ms, 32: 1.68 ms, 48: 1.71 ms for the march of the 2^20-ray batch)
 constexpr uint32_t COUNT_STEP_BURST = 24;
 
-#ifndef SRF_COUNT_WAVES_PER_EU
+// five wavefronts a SIMD: 102 registers a lane, which the counting march just fits
 #define SRF_COUNT_WAVES_PER_EU 5
-#endif
 // counting sort of one chunk of ray indices by ray_chunk_key_body; the order inside a bin is whatever the atomics give
 __global__ void __launch_bounds__(RAY_CHUNK_BINS) k_ray_order(Params P, CountArgs A, uint32_t* __restrict__ order) {
 	__shared__ uint32_t bins[RAY_CHUNK_BINS];   // one thread per bin
@@ -161,10 +160,7 @@ __global__ void __launch_bounds__(256) k_train_keep(uint32_t n_rays, uint32_t n_
 // yields the t of every sample, and drops t and its own number into the sample's slot; then consecutive lanes take
 // consecutive slots, compute what the sample stores (warp, cell, step) and write it, so that the per-sample work
 // is spread evenly whatever the rays' sample counts are, and the stores of a wavefront are contiguous.
-#ifndef SRF_WRITE_WINDOW
-#define SRF_WRITE_WINDOW 1024
-#endif
-constexpr uint32_t WRITE_WINDOW = SRF_WRITE_WINDOW;
+constexpr uint32_t WRITE_WINDOW = 1024;
 
 struct WindowEmit {
 	float* win_t; uint8_t* win_ray;
