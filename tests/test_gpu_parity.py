@@ -516,6 +516,39 @@ def test_render_marches_through_the_one_ray_per_wavefront_march(gpu, orc, config
         assert np.array_equal(pay.cpu().numpy().view(O.PAYLOAD_DTYPE), o_pay) and np.array_equal(g_coords.cpu().numpy(), o_coords)
 
 
+@pytest.mark.parametrize("variant", ["log_stepping", "original_stepping_cone", "reciprocal_grid", "no_pixel_snap"])
+def test_one_ray_per_wavefront_march_under_other_sampler_settings(gpu, orc, variant, monkeypatch):
+    """the same forced hand-over with stepping rules whose 64 steps at once go through calc_dt step by step, on a random bitfield"""
+    torch = gpu
+    monkeypatch.setenv("SRF_MARCH_PARK_ALL", "1")
+    from sphericalrf_amd import api, scene
+    w = scene.workload(2, 0.25)
+    cfg = dict(w["sampler"], num_cascades=2, **SAMPLER_VARIANTS[variant])
+    p = helpers.oracle_params(orc, cfg)
+    rng = np.random.default_rng(7)
+    s = api.OccupancySampler(cfg)
+    monkeypatch.delenv("SRF_MARCH_PARK_ALL")
+    grid = (rng.random(p.n_total) < 0.02).astype(np.float32)
+    bf, _ = orc.update_grid_bitfield(p, grid)
+    s.set_density_grid(torch.from_numpy(grid).cuda())
+    s.update_grid_bitfield()
+    res, cam = w["resolution"], w["cameras"][0]
+    n = res[0] * res[1]
+    table = scene.field_table(1024, 3)
+    table[:, 3] *= 10
+    want_frame, want_ns, _ = orc.render_frame(p, orc.make_field(table, 5), bf, res, w["focal"], (0.5, 0.5), cam, transmittance_threshold=1e-4, train_in_linear_colors=True)
+    m = api.RayMarcher(dict(train_in_linear_color=True, transmittance_threshold=1e-4))
+    frame, fns = torch.ones((res[1], res[0], 4), device="cuda"), torch.zeros(n, dtype=torch.int32, device="cuda")
+    s.render_frame_fused(m, api.Field(torch.from_numpy(table).cuda(), 5), res, w["focal"], (0.5, 0.5), cam, frame, fns)
+    assert np.array_equal(u32(fns).reshape(res[1], res[0]), want_ns) and np.array_equal(frame.cpu().numpy(), want_frame)
+    assert (want_ns > 0).mean() > 0.2
+    pay = torch.zeros(n * 40, dtype=torch.uint8, device="cuda")
+    s.generate_rays_from_camera_matrix(res, w["focal"], (0.5, 0.5), cam, pay)
+    o_pay = orc.init_rays_with_payload(p, res, w["focal"], (0.5, 0.5), cam)
+    orc.advance_pos(p, o_pay, bf)
+    assert np.array_equal(pay.cpu().numpy().view(O.PAYLOAD_DTYPE), o_pay)
+
+
 @pytest.mark.parametrize("res", [(37, 21), (8, 8), (9, 70), (131, 5), (1, 1)])
 def test_fused_frame_sizes_that_do_not_fill_their_pixel_tiles(gpu, orc, res):
     """the fused frame hands 8 x 8 pixel tiles to its wavefronts: widths and heights that leave tiles partly outside the frame"""
