@@ -61,11 +61,14 @@ int srf_render_frame(srf_sampler_t* s, srf_marcher_t* m, const srf_frame_args* a
 	uint32_t* counters = (uint32_t*)(w + 3 * pay_bytes + 3 * col_bytes + coord_bytes + net_bytes);     // [0] alive, [1] hit
 
 	// testbed.cu:502-518
-	SRF_HIP(hipMemsetAsync(frame_buffer, 0, (size_t)n_pixels * 16, st));
+	rc = fill_u32(frame_buffer, (size_t)n_pixels * 4, 0u, st);
+	if (rc != SRF_OK) return rc;
 	rc = srf_sampler_generate_rays_from_camera_matrix(s, a->resolution, a->focal_length, a->principal_point, a->camera_matrix, pay[0], a->spp, st);
 	if (rc != SRF_OK) return rc;
-	SRF_HIP(hipMemsetAsync(col[0], 0, (size_t)n_pixels * 16, st));
-	SRF_HIP(hipMemsetAsync(counters + 1, 0, 4, st));
+	rc = fill_u32(col[0], (size_t)n_pixels * 4, 0u, st);
+	if (rc != SRF_OK) return rc;
+	rc = fill_u32(counters + 1, 1, 0u, st);
+	if (rc != SRF_OK) return rc;
 
 	srf_render_args ra;
 	ra.padded_output_width = a->padded_output_width;
