@@ -241,7 +241,8 @@ __global__ void __launch_bounds__(128) k_init_rays(Params P, PixelArgs A, srf_ra
 // stretches side by side.
 // A ray that crawls (an empty cell and nothing to skip at every probe: it runs along occupied blocks) costs a round of dependent
 // loads a step, and when it is one of the last few rays of its wavefront nothing hides them: such rays alone kept a frame of the
-// bounded-object workload alive four times longer than its average wavefront.  A wavefront down to PARK_MAX_LANES rays therefore
+// bounded-object workload alive four times longer than its average wavefront.  A wavefront down to PARK_MAX_LANES rays (16: 8
+// leaves a seventh of that frame's time on the table, 32 gains nothing more) therefore
 // parks those that have crawled PARK_CRAWL probes in a row: the lane's state goes to a queue as it stands, and k_march_wide
 // carries each parked ray on, one ray a wavefront.  There a crawling ray is taken through its next 64 steps at once: every lane
 // follows the chain of t (it has to be followed step by step) and keeps the value before its own step, looks that position up, and
@@ -249,7 +250,7 @@ __global__ void __launch_bounds__(128) k_init_rays(Params P, PixelArgs A, srf_ra
 // ray's state moves, so the march's outcome is the one of probing step by step.
 // (settled on the render workloads: parking after 16 or 32 probes costs the frames without such rays 5 to 10 % in rays that
 // would have stopped crawling soon; wide rounds inside the march kernel itself cost them more than that in registers)
-constexpr uint32_t PARK_MAX_LANES = 8, PARK_CRAWL = 64;
+constexpr uint32_t PARK_MAX_LANES = 16, PARK_CRAWL = 64;
 struct MarchPark { void* slots; uint32_t* count; uint32_t* next_count; uint32_t capacity, max_lanes, min_crawl; };
 
 __device__ __forceinline__ float lane_value_f32(float v, uint32_t uniform_lane) { return srf_u2f(lane_value_u32(srf_f2u(v), uniform_lane)); }
