@@ -549,6 +549,38 @@ def test_one_ray_per_wavefront_march_under_other_sampler_settings(gpu, orc, vari
     assert np.array_equal(pay.cpu().numpy().view(O.PAYLOAD_DTYPE), o_pay)
 
 
+@pytest.mark.parametrize("n", [1, 63, 1024, 1025, 70001])
+def test_ray_compaction_keeps_the_source_order_and_continues_the_counters(gpu, n):
+    """compact_rays_kernel (internal/testbed.cu:423-446) with the positions handed out in source order: live rays to the destination,
+    dead rays with visible alpha to the final buffers, both behind what the counters already hold; sizes around the block of 1024"""
+    torch = gpu
+    from sphericalrf_amd import api
+    rng = np.random.default_rng(n)
+    pay = np.zeros(n, O.PAYLOAD_DTYPE)
+    pay["alive"] = rng.random(n) < 0.4
+    pay["idx"] = np.arange(n)
+    pay["t"] = rng.random(n).astype(np.float32)
+    pay["o"] = rng.random((n, 3)).astype(np.float32)
+    rgba = rng.random((n, 4)).astype(np.float32)
+    rgba[rng.random(n) < 0.5, 3] = 0.0005          # dead and invisible: dropped
+    m = api.RayMarcher(dict())
+    a0, f0 = 5, 7
+    room = n + 8
+    dst_p, fin_p = torch.zeros(room * 40, dtype=torch.uint8, device="cuda"), torch.zeros(room * 40, dtype=torch.uint8, device="cuda")
+    dst_c, fin_c = torch.zeros((room, 4), device="cuda"), torch.zeros((room, 4), device="cuda")
+    na, nf = torch.full((1,), a0, dtype=torch.int32, device="cuda"), torch.full((1,), f0, dtype=torch.int32, device="cuda")
+    api.compact_rays(m, n, torch.from_numpy(pay.view(np.uint8)).cuda(), torch.from_numpy(rgba).cuda(), dst_p, dst_c, fin_p, fin_c, na, nf)
+    alive = pay["alive"] == 1
+    final = ~alive & (rgba[:, 3] > 0.001)
+    assert int(na.item()) == a0 + alive.sum() and int(nf.item()) == f0 + final.sum()
+    got_p, got_f = dst_p.cpu().numpy().view(O.PAYLOAD_DTYPE), fin_p.cpu().numpy().view(O.PAYLOAD_DTYPE)
+    assert got_p[a0:a0 + alive.sum()].tobytes() == pay[alive].tobytes() and np.array_equal(dst_c.cpu().numpy()[a0:a0 + alive.sum()], rgba[alive])
+    assert got_f[f0:f0 + final.sum()].tobytes() == pay[final].tobytes() and np.array_equal(fin_c.cpu().numpy()[f0:f0 + final.sum()], rgba[final])
+    # nothing before the counters' old values or behind the new ones is touched
+    assert not got_p[:a0].view(np.uint8).any() and not got_p[a0 + alive.sum():].view(np.uint8).any()
+    assert not got_f[:f0].view(np.uint8).any() and not got_f[f0 + final.sum():].view(np.uint8).any()
+
+
 @pytest.mark.parametrize("res", [(37, 21), (8, 8), (9, 70), (131, 5), (1, 1)])
 def test_fused_frame_sizes_that_do_not_fill_their_pixel_tiles(gpu, orc, res):
     """the fused frame hands 8 x 8 pixel tiles to its wavefronts: widths and heights that leave tiles partly outside the frame"""
