@@ -220,9 +220,10 @@ def bench_render(torch, api, scene, config_id, steps, warmup, n_frames=2):
                 samples_per_s=total / sec, loop_ms_per_frame=loop_sec * 1e3, loop_rounds_last_frame=rounds["n"], occupied_bits=occ, frames_in_workload=len(cams))
 
 
-def bench_grid_update(torch, api, scene, steps, warmup):
+def bench_grid_update(torch, api, scene, steps, warmup, cell_order=False):
     w = scene.workload(5)
     s = api.OccupancySampler(w["sampler"])
+    s.set_grid_sample_order(cell_order)
     s.init(1, w["resolution"], w["focal"], (0.5, 0.5), None, None, api.Pcg32(43))
     n_total = int(s.n_total_elements)
     pos = torch.zeros((n_total, 3), device="cuda")
@@ -255,7 +256,7 @@ def bench_grid_update(torch, api, scene, steps, warmup):
     avg = {k: sum(v) / len(v) for k, v in parts.items()}
     import numpy as np
     occ = float(np.unpackbits(s.density_grid_bitfield.cpu().numpy()).mean())
-    return dict(workload="grid_update_5", cells=n_total, ms_per_update=sec * 1e3, parts_ms=avg, occupied_bits=occ,
+    return dict(workload="grid_update_5" + ("_cell_order" if cell_order else ""), cells=n_total, ms_per_update=sec * 1e3, parts_ms=avg, occupied_bits=occ,
                 update_grid_gbs=EMA_BYTES_PER_CELL * n_total / (avg["update_grid"] * 1e-3) / 1e9,
                 bitfield_gbs=BITFIELD_BYTES_PER_CELL * n_total / (avg["update_grid_bitfield"] * 1e-3) / 1e9)
 
@@ -332,6 +333,7 @@ def main():
             log(json.dumps(extras[-1]))
             torch.cuda.empty_cache()
         extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1))
+        extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1, cell_order=True))
         extras.append(bench_grid_sample_draws(torch, api, scene, max(2, args.steps // 2)))
         log(json.dumps(extras[-1]))
         out["extras"] = extras

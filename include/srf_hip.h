@@ -156,6 +156,16 @@ int  srf_ray_sphere_bounds(uint32_t n_rays, const float* rays, const float cente
 /* Testbed::load_snapshot, internal/testbed.cu:167: overwrite density_grid (n_total_elements floats, device) */
 int  srf_sampler_set_density_grid(srf_sampler_t* s, const float* density_grid, void* stream);
 
+/* No counterpart in the reference: the order in which srf_sampler_sample_positions_from_grid hands the uniform points over.
+ * 0 (default): the reference's, point i in entry i.  1, cell order: with a power-of-two cell count n_cells (at least 2048) the
+ * first n_cells * floor(n_uniform / n_cells) entries hold the same points sorted by the cell they fall in, entry
+ * t = m * n_cells + v holding point i = ((v * A' - step * n_uniform) mod n_cells) + m * n_cells (A' the inverse of 56924617
+ * modulo 2^32, step the number of srf_sampler_update_grid calls so far); every later entry is as in order 0.
+ * srf_sampler_update_grid, given densities and indices in that same order, then combines those entries per cell without
+ * sorting them (it checks each entry's index, so arrays in any other order still give the right grid, only slower).
+ * The set of points, their positions and indices and the grid that results are those of order 0. */
+int  srf_sampler_set_grid_sample_order(srf_sampler_t* s, int32_t cell_order);
+
 /* OccupancySampler::sample_positions_from_grid, occupancy_sampler.cu:980-1029.
  * grid_positions: (n_uniform + n_nonuniform) x 3 floats; grid_indices: as many uint32. */
 int  srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform_positions, uint32_t n_nonuniform_positions,

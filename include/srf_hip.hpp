@@ -95,6 +95,7 @@ public:
 	void update_grid_bitfield(void* stream) { check(srf_sampler_update_grid_bitfield(m_impl, stream)); }
 	// snapshot load (testbed.cu:158-168): the caller's grid replaces density_grid
 	void set_ray_sphere_bound(const float center[3], float radius) { check(srf_sampler_set_ray_sphere_bound(m_impl, center, radius)); }
+	void set_grid_sample_order(bool cell_order) { check(srf_sampler_set_grid_sample_order(m_impl, cell_order ? 1 : 0)); }
 	void set_density_grid(const float* density_grid_device, void* stream) { check(srf_sampler_set_density_grid(m_impl, density_grid_device, stream)); }
 
 	// occupancy_sampler.cu:1090-1143; sample_t / sample_dt / sample_cell are optional extras (NULL to skip)

@@ -107,7 +107,7 @@ SYMBOLS = [
     "srf_sampler_config_default", "srf_sampler_create", "srf_sampler_destroy", "srf_sampler_get_info", "srf_sampler_set_runtime",
     "srf_sampler_init", "srf_sampler_set_density_grid", "srf_sampler_sample_positions_from_grid", "srf_sampler_update_grid",
     "srf_sampler_update_grid_bitfield", "srf_sampler_sample_coords_from_dataset", "srf_sampler_generate_rays_from_camera_matrix",
-    "srf_sampler_generate_coords_from_rays", "srf_sampler_set_ray_sphere_bound", "srf_ray_sphere_bounds",
+    "srf_sampler_generate_coords_from_rays", "srf_sampler_set_ray_sphere_bound", "srf_ray_sphere_bounds", "srf_sampler_set_grid_sample_order",
     "srf_marcher_config_default", "srf_marcher_create", "srf_marcher_destroy", "srf_marcher_get_config", "srf_marcher_set_config",
     "srf_marcher_volume_rendering_with_loss_and_gradient", "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc", "srf_marcher_sync_check", "srf_marcher_volume_rendering",
     "srf_compact_rays", "srf_shade", "srf_fill_rollover", "srf_fill_rollover_and_rescale",
@@ -149,6 +149,7 @@ def load():
     L.srf_sampler_init.argtypes = [vp, u32, P(i32 * 2), P(f32 * 2), P(f32 * 2), vp, P(Pcg32), vp]
     L.srf_sampler_set_density_grid.argtypes = [vp, vp, vp]
     L.srf_sampler_set_ray_sphere_bound.argtypes = [vp, P(f32 * 3), f32]
+    L.srf_sampler_set_grid_sample_order.argtypes = [vp, i32]
     L.srf_ray_sphere_bounds.argtypes = [u32, vp, P(f32 * 3), f32, vp, vp, vp]
     L.srf_sampler_sample_positions_from_grid.argtypes = [vp, u32, u32, vp, vp, vp]
     L.srf_sampler_update_grid.argtypes = [vp, u32, u32, vp, i32, vp, i32, vp]

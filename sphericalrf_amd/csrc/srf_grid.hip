@@ -47,15 +47,16 @@ __global__ void __launch_bounds__(256) k_mark_untrained(Params P, uint32_t n_tot
 __global__ void __launch_bounds__(256) k_generate_grid_samples(Params P, uint32_t n_elements, Pcg32 rng, uint32_t step,
                                                                 const float* __restrict__ grid_in, float thresh,
                                                                 float* __restrict__ positions, uint32_t* __restrict__ indices, const uint32_t* __restrict__ above,
-                                                                uint32_t tries_at_once) {
+                                                                uint32_t tries_at_once, uint32_t first) {
 	// the generator's skip-ahead maps, one hexadecimal digit each, worked out once per workgroup
 	__shared__ uint64_t skip_m[128], skip_p[128];
 	if (threadIdx.x < 128) pcg_skip16_entry(rng, threadIdx.x, &skip_m[threadIdx.x], &skip_p[threadIdx.x]);
 	__syncthreads();
 	// a workgroup takes several runs of 256 points: the launch is then a few thousand groups instead of one per run
-	const uint32_t n_runs = (n_elements + 255u) / 256u;
+	// the points from `first` on
+	const uint32_t n_runs = (n_elements - first + 255u) / 256u;
 	for (uint32_t run = blockIdx.x; run < n_runs; run += gridDim.x) {
-		const uint32_t i = run * 256u + threadIdx.x;
+		const uint32_t i = first + run * 256u + threadIdx.x;
 		if (i < n_elements) grid_sample_body(i, P, n_elements, rng, step, grid_in, thresh, positions, indices, above, nullptr, tries_at_once, skip_m, skip_p);
 	}
 }
@@ -70,7 +71,8 @@ __global__ void __launch_bounds__(256) k_generate_grid_samples(Params P, uint32_
 __global__ void __launch_bounds__(256) k_generate_grid_samples_by_cell(Params P, uint32_t n_elements, Pcg32 rng, uint32_t step,
                                                                         const float* __restrict__ grid_in, float thresh,
                                                                         Float4* __restrict__ staged, const uint32_t* __restrict__ above,
-                                                                        uint32_t tries_at_once, uint32_t a_inverse, uint32_t log2_cells) {
+                                                                        uint32_t tries_at_once, uint32_t a_inverse, uint32_t log2_cells,
+                                                                        float* __restrict__ positions, uint32_t* __restrict__ indices) {
 	__shared__ uint64_t skip_m[128], skip_p[128];
 	if (threadIdx.x < 128) pcg_skip16_entry(rng, threadIdx.x, &skip_m[threadIdx.x], &skip_p[threadIdx.x]);
 	__syncthreads();
@@ -83,7 +85,9 @@ __global__ void __launch_bounds__(256) k_generate_grid_samples_by_cell(Params P,
 	Vec3 pos;
 	uint32_t idx;
 	grid_sample_point((uint32_t)i, P, n_elements, rng, step, grid_in, thresh, &pos, &idx, above, nullptr, tries_at_once, skip_m, skip_p);
-	staged[t] = mk4(pos.x, pos.y, pos.z, srf_u2f(idx));
+	// staged == NULL: the caller takes the points in this order (entry t of its arrays is thread t's point)
+	if (staged) staged[t] = mk4(pos.x, pos.y, pos.z, srf_u2f(idx));
+	else { st3(positions + 3 * (size_t)t, pos); indices[t] = idx; }
 }
 
 __global__ void __launch_bounds__(256) k_grid_samples_to_point_order(uint32_t n_cells, uint32_t n_elements, uint32_t step, uint32_t log2_cells,
@@ -164,6 +168,53 @@ __global__ void __launch_bounds__(256) k_splat_slabs(uint32_t n_elements, uint32
 	__syncthreads();
 	const uint32_t first = slab << SPLAT_SLAB_BITS;
 	for (uint32_t j = threadIdx.x; j < SPLAT_SLAB_CELLS; j += 256u) if (first + j < n_total) grid_current_bits[first + j] = tile[j];
+}
+
+// The splat of samples that arrive dealt by cell (k_generate_grid_samples_by_cell's order, taken as it is by the caller):
+// entry t = m n_cells + v lies in cell (v + 96925573) mod n_cells of some cascade when its point's first try passed, as nearly
+// all tries against the -0.01 threshold do.  A workgroup owns DEALT_CELLS consecutive cells of every cascade, reads the entries
+// that the dealing puts there (one contiguous stretch per m, two where it wraps), combines them in LDS and writes its cells
+// of every cascade: no sort and no device atomics.  Every entry is checked against the place it is read from; one that lies
+// elsewhere (a later try, or arrays that are not in this order at all) goes to a list that k_splat_listed applies afterwards.
+// MERGE: the cells already hold the splat of other samples (those not in this order), so the result is the larger of both.
+constexpr uint32_t DEALT_CELLS = 2048;
+constexpr uint32_t DEALT_FIRST_CELL = 96925573u;      // the constant of the candidate-cell hash (grid_sample_tries)
+template <bool HALF, bool MERGE>
+__global__ void __launch_bounds__(256) k_splat_dealt(uint32_t n_cells, uint32_t log2_cells, uint32_t n_cascades, uint32_t n_blocks_m, const uint32_t* __restrict__ indices,
+                                                      uint32_t width, const void* __restrict__ densities, int act, float min_cone_stepsize,
+                                                      uint32_t* __restrict__ grid_current_bits, uint32_t* __restrict__ list_count, U2* __restrict__ list) {
+	extern __shared__ uint32_t tiles[];                      // [cascade][DEALT_CELLS]
+	const uint32_t mask = n_cells - 1u;
+	const uint32_t cell0 = blockIdx.x * DEALT_CELLS;
+	for (uint32_t j = threadIdx.x; j < n_cascades * DEALT_CELLS; j += 256u) tiles[j] = 0u;
+	__syncthreads();
+	for (uint32_t m = 0; m < n_blocks_m; ++m) {
+		for (uint32_t k = threadIdx.x; k < DEALT_CELLS; k += 256u) {
+			const uint32_t cell = cell0 + k;
+			const size_t t = ((size_t)m << log2_cells) + ((cell - DEALT_FIRST_CELL) & mask);
+			const uint32_t idx = indices[t];
+			const float sigma = act_density(net_load<HALF>(densities, t * width), act);
+			const uint32_t bits = srf_f2u(sigma * min_cone_stepsize);
+			if (bits == 0u) continue;                        // cannot raise a cell
+			const uint32_t level = idx >> log2_cells;
+			if ((idx & mask) == cell && level < n_cascades) atomicMax(&tiles[level * DEALT_CELLS + k], bits);
+			else { const uint32_t at = atomicAdd(list_count, 1u); U2 e; e.x = idx; e.y = bits; list[at] = e; }
+		}
+	}
+	__syncthreads();
+	for (uint32_t j = threadIdx.x; j < n_cascades * DEALT_CELLS; j += 256u) {
+		const size_t at = (size_t)(j / DEALT_CELLS) * n_cells + cell0 + (j % DEALT_CELLS);
+		uint32_t v = tiles[j];
+		if (MERGE) { const uint32_t old = grid_current_bits[at]; v = old > v ? old : v; }
+		grid_current_bits[at] = v;
+	}
+}
+__global__ void __launch_bounds__(256) k_splat_listed(const uint32_t* __restrict__ list_count, const U2* __restrict__ list, uint32_t n_total, uint32_t* __restrict__ grid_current_bits) {
+	const uint32_t n = *list_count;
+	for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+		const U2 e = list[i];
+		if (e.x < n_total) atomicMax(&grid_current_bits[e.x], e.y);
+	}
 }
 
 // occupancy_sampler.cu:214-238 — decayed maximum, four cells per thread
@@ -533,6 +584,14 @@ int srf_sampler_set_density_grid(srf_sampler_t* s, const float* density_grid, vo
 	return SRF_OK;
 }
 
+int srf_sampler_set_grid_sample_order(srf_sampler_t* s, int32_t cell_order) {
+	SRF_REQUIRE(s, "srf_sampler_set_grid_sample_order: NULL sampler");
+	SRF_REQUIRE(cell_order == 0 || cell_order == 1, "srf_sampler_set_grid_sample_order: order must be 0 or 1");
+	s->grid_sample_cell_order = cell_order != 0;
+	s->dealt_entries = 0;
+	return SRF_OK;
+}
+
 int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform, uint32_t n_nonuniform,
                                            float* grid_positions, uint32_t* grid_indices, void* stream) {
 	SRF_REQUIRE(s, "srf_sampler_sample_positions_from_grid: NULL sampler");
@@ -567,29 +626,40 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 		above_a = a; above_b = b;
 	}
 	const uint32_t tries = 1;     // looking several candidates up at once (up to 4) has made no measurable difference
-	if (n_uniform) {
-		hipLaunchKernelGGL(k_generate_grid_samples, dim3(div_up(n_uniform, 256) < 16384u ? div_up(n_uniform, 256) : 16384u), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, -0.01f, grid_positions, grid_indices, above_a, 1u);   // nearly every first try passes
+	uint32_t log2_cells = 0;
+	while ((1u << log2_cells) < nc) ++log2_cells;
+	uint32_t inv = 56924617u;                                  // inverse of the hash multiplier modulo 2^32, by Newton's iteration
+	for (int k = 0; k < 5; ++k) inv *= 2u - 56924617u * inv;
+	// Cell order (srf_sampler_set_grid_sample_order): the uniform points of whole multiples of the cell count stay in the order
+	// of the dealing, entry t = m n_cells + v holding the point whose (i + step n) A mod n_cells is v; srf_sampler_update_grid
+	// then splats them without sorting.  The other points follow in their own order.
+	const uint32_t n_dealt = s->grid_sample_cell_order && (nc & (nc - 1u)) == 0u && nc >= DEALT_CELLS ? n_uniform / nc * nc : 0u;
+	s->dealt_entries = n_dealt;
+	if (n_dealt) {
+		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(n_dealt / 256u), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, -0.01f, (Float4*)nullptr, above_a, 1u, inv, log2_cells, grid_positions, grid_indices);
+		SRF_LAUNCH_CHECK();
+	}
+	if (n_uniform > n_dealt) {
+		const uint32_t runs = div_up(n_uniform - n_dealt, 256);
+		hipLaunchKernelGGL(k_generate_grid_samples, dim3(runs < 16384u ? runs : 16384u), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, -0.01f, grid_positions, grid_indices, above_a, 1u, n_dealt);   // nearly every first try passes
 		SRF_LAUNCH_CHECK();
 	}
 	pcg_advance(s->rng, 1ull << 32);
 	float* positions_b = grid_positions + 3 * (size_t)n_uniform;
 	uint32_t* indices_b = grid_indices + n_uniform;
 	if (by_cell) {
-		uint32_t log2_cells = 0;
-		while ((1u << log2_cells) < nc) ++log2_cells;
-		uint32_t inv = 56924617u;                                  // inverse of the hash multiplier modulo 2^32, by Newton's iteration
-		for (int k = 0; k < 5; ++k) inv *= 2u - 56924617u * inv;
 		Float4* staged = (Float4*)((char*)s->ws.ptr + 2 * table_bytes);
 		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3((uint32_t)(dealt_threads / 256u)), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, staged, above_b, tries, inv, log2_cells);
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, staged, above_b, tries, inv, log2_cells, (float*)nullptr, (uint32_t*)nullptr);
 		SRF_LAUNCH_CHECK();
 		hipLaunchKernelGGL(k_grid_samples_to_point_order, dim3(div_up(n_nonuniform, 256)), dim3(256), 0, st, nc, n_nonuniform, s->i_step, log2_cells,
 		                   (const Float4*)staged, positions_b, indices_b);
 		SRF_LAUNCH_CHECK();
 	} else if (n_nonuniform) {
 		hipLaunchKernelGGL(k_generate_grid_samples, dim3(div_up(n_nonuniform, 256) < 16384u ? div_up(n_nonuniform, 256) : 16384u), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, positions_b, indices_b, above_b, tries);
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, positions_b, indices_b, above_b, tries, 0u);
 		SRF_LAUNCH_CHECK();
 	}
 	pcg_advance(s->rng, 1ull << 32);
@@ -606,40 +676,73 @@ int srf_sampler_update_grid(srf_sampler_t* s, uint32_t n_total_positions, uint32
 	SRF_REQUIRE(densities_dtype == SRF_DTYPE_F16 || densities_dtype == SRF_DTYPE_F32, "srf_sampler_update_grid: unknown dtype");
 	SRF_REQUIRE(density_activation >= SRF_ACT_NONE && density_activation <= SRF_ACT_EXPONENTIAL, "srf_sampler_update_grid: unknown activation");
 	hipStream_t st = (hipStream_t)stream;
-	bool sorted_splat = n_total_positions >= SPLAT_SORT_MIN;
-	if (s->force_splat_sort >= 0) sorted_splat = s->force_splat_sort != 0 && n_total_positions != 0;
-	int rc = sorted_splat ? SRF_OK : fill_u32(s->density_grid_current, s->n_total, 0u, st);
+	const bool half = densities_dtype == SRF_DTYPE_F16;
+	const uint32_t nc = s->P.n_cells;
+	// the leading entries that the last srf_sampler_sample_positions_from_grid left in cell order (every one of them is checked
+	// where it is used: arrays in another order cost time, not correctness), and the others
+	uint32_t n_dealt = s->grid_sample_cell_order && s->dealt_entries < n_total_positions ? s->dealt_entries : (s->grid_sample_cell_order ? n_total_positions : 0u);
+	n_dealt = (nc & (nc - 1u)) == 0u && nc >= DEALT_CELLS ? n_dealt / nc * nc : 0u;
+	const uint32_t n = n_total_positions - n_dealt;
+	const uint32_t* rest_indices = grid_indices ? grid_indices + n_dealt : nullptr;
+	const void* rest_densities = grid_densities ? (const char*)grid_densities + (size_t)n_dealt * padded_output_width * (half ? 2 : 4) : nullptr;
+	bool sorted_splat = n >= SPLAT_SORT_MIN;
+	if (s->force_splat_sort >= 0) sorted_splat = s->force_splat_sort != 0 && n != 0;
+	// who clears the cells: the slabs of the sorted splat or the dealt splat, which write every cell, or else a fill
+	int rc = sorted_splat || n_dealt ? SRF_OK : fill_u32(s->density_grid_current, s->n_total, 0u, st);
 	if (rc != SRF_OK) return rc;
-	if (sorted_splat) {
-		const uint32_t n = n_total_positions;
-		int end_bit = (int)SPLAT_SLAB_BITS + 1;
-		while (end_bit < 32 && (1ull << end_bit) < (unsigned long long)s->n_total) ++end_bit;
-		size_t temp_bytes = 0;
+	int end_bit = (int)SPLAT_SLAB_BITS + 1;
+	while (end_bit < 32 && (1ull << end_bit) < (unsigned long long)s->n_total) ++end_bit;
+	size_t temp_bytes = 0;
+	if (sorted_splat)
 		SRF_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, (const uint32_t*)nullptr, (uint32_t*)nullptr, (const uint32_t*)nullptr, (uint32_t*)nullptr,
 		                                           (int)n, (int)SPLAT_SLAB_BITS, end_bit, st));
-		const size_t arr = align_up((size_t)n * 4, 256);
-		rc = s->ws.reserve(3 * arr + temp_bytes);
-		if (rc != SRF_OK) return rc;
+	const size_t arr = sorted_splat ? align_up((size_t)n * 4, 256) : 0;
+	const size_t sort_bytes = sorted_splat ? align_up(3 * arr + temp_bytes, 256) : 0;
+	const size_t list_bytes = n_dealt ? 256 + (size_t)n_dealt * sizeof(U2) : 0;
+	rc = s->ws.reserve(sort_bytes + list_bytes);
+	if (rc != SRF_OK) return rc;
+	if (sorted_splat) {
 		uint32_t* thick = (uint32_t*)s->ws.ptr;
 		uint32_t* cells_sorted = (uint32_t*)((char*)s->ws.ptr + arr);
 		uint32_t* thick_sorted = (uint32_t*)((char*)s->ws.ptr + 2 * arr);
 		void* temp = (char*)s->ws.ptr + 3 * arr;
-		if (densities_dtype == SRF_DTYPE_F16)
-			hipLaunchKernelGGL(k_splat_values<true>, dim3(div_up(n, 256)), dim3(256), 0, st, n, padded_output_width, grid_densities, density_activation, s->P.min_cone_stepsize, thick);
+		if (half)
+			hipLaunchKernelGGL(k_splat_values<true>, dim3(div_up(n, 256)), dim3(256), 0, st, n, padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, thick);
 		else
-			hipLaunchKernelGGL(k_splat_values<false>, dim3(div_up(n, 256)), dim3(256), 0, st, n, padded_output_width, grid_densities, density_activation, s->P.min_cone_stepsize, thick);
+			hipLaunchKernelGGL(k_splat_values<false>, dim3(div_up(n, 256)), dim3(256), 0, st, n, padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, thick);
 		SRF_LAUNCH_CHECK();
-		SRF_HIP(hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, grid_indices, cells_sorted, (const uint32_t*)thick, thick_sorted, (int)n, (int)SPLAT_SLAB_BITS, end_bit, st));
+		SRF_HIP(hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, rest_indices, cells_sorted, (const uint32_t*)thick, thick_sorted, (int)n, (int)SPLAT_SLAB_BITS, end_bit, st));
 		hipLaunchKernelGGL(k_splat_slabs, dim3(div_up(s->n_total, SPLAT_SLAB_CELLS)), dim3(256), 0, st, n, s->n_total, (const uint32_t*)cells_sorted,
 		                   (const uint32_t*)thick_sorted, (uint32_t*)s->density_grid_current);
 		SRF_LAUNCH_CHECK();
-	} else if (n_total_positions) {
-		if (densities_dtype == SRF_DTYPE_F16)
-			hipLaunchKernelGGL(k_splat_grid_samples<true>, dim3(div_up(n_total_positions, 256)), dim3(256), 0, st, n_total_positions, grid_indices,
-			                   padded_output_width, grid_densities, density_activation, s->P.min_cone_stepsize, s->density_grid_current);
+	}
+	uint32_t* list_count = (uint32_t*)((char*)s->ws.ptr + sort_bytes);
+	U2* list = (U2*)((char*)s->ws.ptr + sort_bytes + 256);
+	if (n_dealt) {
+		rc = fill_u32(list_count, 1, 0u, st);
+		if (rc != SRF_OK) return rc;
+		uint32_t log2_cells = 0;
+		while ((1u << log2_cells) < nc) ++log2_cells;
+		const dim3 grid(nc / DEALT_CELLS), block(256);
+		const size_t lds = (size_t)s->P.n_cascades * DEALT_CELLS * sizeof(uint32_t);
+#define SRF_DEALT(H, M) hipLaunchKernelGGL((k_splat_dealt<H, M>), grid, block, lds, st, nc, log2_cells, s->P.n_cascades, n_dealt / nc, grid_indices, padded_output_width, grid_densities, \
+                                           density_activation, s->P.min_cone_stepsize, (uint32_t*)s->density_grid_current, list_count, list)
+		if (half) { if (sorted_splat) SRF_DEALT(true, true); else SRF_DEALT(true, false); }
+		else { if (sorted_splat) SRF_DEALT(false, true); else SRF_DEALT(false, false); }
+#undef SRF_DEALT
+		SRF_LAUNCH_CHECK();
+	}
+	if (!sorted_splat && n) {
+		if (half)
+			hipLaunchKernelGGL(k_splat_grid_samples<true>, dim3(div_up(n, 256)), dim3(256), 0, st, n, rest_indices,
+			                   padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, s->density_grid_current);
 		else
-			hipLaunchKernelGGL(k_splat_grid_samples<false>, dim3(div_up(n_total_positions, 256)), dim3(256), 0, st, n_total_positions, grid_indices,
-			                   padded_output_width, grid_densities, density_activation, s->P.min_cone_stepsize, s->density_grid_current);
+			hipLaunchKernelGGL(k_splat_grid_samples<false>, dim3(div_up(n, 256)), dim3(256), 0, st, n, rest_indices,
+			                   padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, s->density_grid_current);
+		SRF_LAUNCH_CHECK();
+	}
+	if (n_dealt) {
+		hipLaunchKernelGGL(k_splat_listed, dim3(1024), dim3(256), 0, st, (const uint32_t*)list_count, (const U2*)list, s->n_total, (uint32_t*)s->density_grid_current);
 		SRF_LAUNCH_CHECK();
 	}
 	const uint32_t n_vec4 = s->n_total / 4;

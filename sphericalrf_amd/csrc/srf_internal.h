@@ -60,6 +60,8 @@ struct srf_sampler {
 	// SRF_COUNT_PROBE_BUDGET = lookups after which the counting march parks a ray (0: never)
 	int      force_splat_sort, force_sample_bits, force_sample_by_cell;
 	uint32_t count_probe_budget;
+	bool     grid_sample_cell_order = false;   // srf_sampler_set_grid_sample_order
+	uint32_t dealt_entries = 0;                // leading entries the last sample_positions_from_grid left in cell order
 	srf::Workspace ws;
 	srf::Workspace park_ws;          // queue of the rays the render marches hand to their one-ray-per-wavefront march
 	uint32_t* park_counts = nullptr; // two counters of that queue, used in turn: a march clears the one the next march will use

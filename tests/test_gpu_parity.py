@@ -120,6 +120,74 @@ def test_grid_maintenance(gpu, orc, N, C, large_batch_path, monkeypatch):
     assert s.i_step == 3
 
 
+# The opt-in cell order of the uniform points: the entries are the reference's points in the documented permutation, and
+# update_grid, given densities and indices in that order, leaves the grid the oracle gets from the reference's order.
+# Step 0: every point in cell order (a whole multiple of the cell count).  Step 1: a grid with masked cells, so that some
+# uniform points settle on a later try (their entries do not lie in the cell the order puts them in), two and a half
+# multiples plus a non-uniform draw (the entries that follow in the reference's order go through the splat of small or, forced,
+# of large batches).  Step 2: fewer points than cells (nothing is in cell order).  Step 3: arrays handed to update_grid in
+# the reference's order although the sampler drew them in cell order (every entry fails its check; the grid is still right).
+@pytest.mark.parametrize("large_batch_path", ["0", "1"])
+@pytest.mark.parametrize("N,C", [((64, 32, 32), 5), ((128, 128, 128), 2)])
+def test_grid_samples_in_cell_order(gpu, orc, N, C, large_batch_path, monkeypatch):
+    torch = gpu
+    monkeypatch.setenv("SRF_SPLAT_SORT", large_batch_path)
+    monkeypatch.setenv("SRF_GRID_SAMPLE_BITS", large_batch_path)
+    from sphericalrf_amd import api
+    cfg = dict(warping_type="ERP", aabb_scale=16, grid_size=N, num_cascades=C, grid_distribution_type="WarpedSpace_Exp", init_grid_with_mask=False,
+               maximum_marching_steps=256, sampling_type="Disparity", near_distance=0.05, far_distance=10.0)
+    p = helpers.oracle_params(orc, cfg)
+    s = api.OccupancySampler(cfg)
+    s.set_grid_sample_order(True)
+    caller, o_caller = api.Pcg32(44), orc.pcg32(44)
+    s.init(1, (4, 4), (1.0, 1.0), (0.5, 0.5), None, None, caller)
+    o_rng = orc.pcg32(orc.next_uint(o_caller), 1)
+    o_grid = np.zeros(p.n_total, np.float32)
+    rng = np.random.default_rng(2)
+    nc, n_total = int(s.n_grid_elements), p.n_total
+    for step, (n_uni, n_non) in enumerate([(n_total, 0), (2 * nc + nc // 2, nc // 2), (nc // 2, nc // 4), (nc, 100)]):
+        if step == 1:
+            o_grid[rng.random(n_total) < 0.15] = -1.0          # masked cells: a uniform point that draws one tries the next candidate
+            s.set_density_grid(torch.from_numpy(o_grid).cuda())
+        n = n_uni + n_non
+        pos = torch.zeros((n, 3), dtype=torch.float32, device="cuda")
+        idx = torch.zeros(n, dtype=torch.int32, device="cuda")
+        assert s.i_step == step
+        entry_point = s.grid_sample_entry_points(n_uni)
+        n_dealt = n_uni // nc * nc
+        assert entry_point.shape == (n_dealt,) and np.array_equal(np.sort(entry_point), np.arange(n_dealt, dtype=np.uint32))
+        order = np.concatenate([entry_point, np.arange(n_dealt, n, dtype=np.uint32)]).astype(np.int64)
+        s.sample_positions_from_grid(n_uni, n_non, pos, idx)
+        wp1, wi1 = orc.generate_grid_samples(p, n_uni, o_rng, step, o_grid, -0.01)
+        orc.advance(o_rng)
+        wp2, wi2 = orc.generate_grid_samples(p, n_non, o_rng, step, o_grid, p.min_optical_thickness)
+        orc.advance(o_rng)
+        want_idx, want_pos = np.concatenate([wi1, wi2]), np.concatenate([wp1, wp2])
+        assert np.array_equal(u32(idx), want_idx[order])
+        assert np.array_equal(pos.cpu().numpy(), want_pos[order])
+        if step == 1:
+            first_cell = (np.arange(n_dealt, dtype=np.uint64) + 96925573) % nc
+            moved = (want_idx[order][:n_dealt] % nc) != first_cell
+            assert 0.05 < moved.mean() < 0.3                      # the entries that update_grid has to take out of the order
+        dens = np.log1p(np.exp(rng.normal(size=(n, 1)))).astype(np.float16)
+        dens[rng.random(n) < 0.2] = 0                             # samples that raise nothing
+        if step < 3:
+            s.update_grid(n, 1, torch.from_numpy(dens[order]).cuda(), idx, api.ACT_NONE)
+        else:
+            s.update_grid(n, 1, torch.from_numpy(dens).cuda(), torch.from_numpy(want_idx.view(np.int32)).cuda(), api.ACT_NONE)
+        cur = np.zeros(n_total, np.float32)
+        orc.splat_grid_samples(p, want_idx, 1, dens, O.ACT_NONE, cur)
+        orc.ema_grid(cur, p.ema_decay, o_grid)
+        assert np.array_equal(s.density_grid.cpu().numpy(), o_grid)
+    # back to the reference's order
+    s.set_grid_sample_order(False)
+    pos = torch.zeros((n_total, 3), dtype=torch.float32, device="cuda")
+    idx = torch.zeros(n_total, dtype=torch.int32, device="cuda")
+    s.sample_positions_from_grid(n_total, 0, pos, idx)
+    wp1, wi1 = orc.generate_grid_samples(p, n_total, o_rng, 4, o_grid, -0.01)
+    assert np.array_equal(u32(idx), wi1) and np.array_equal(pos.cpu().numpy(), wp1)
+
+
 # probe budget of the counting march: the library's own, never parking a ray, and parking every ray at its first lookup
 # (20000 rays against a queue of 4096: most are refused and carry on, the rest finish in the wide march)
 @pytest.mark.parametrize("budget", [None, "0", "1"])
