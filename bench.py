@@ -220,27 +220,30 @@ def bench_render(torch, api, scene, config_id, steps, warmup, n_frames=2):
                 samples_per_s=total / sec, loop_ms_per_frame=loop_sec * 1e3, loop_rounds_last_frame=rounds["n"], occupied_bits=occ, frames_in_workload=len(cams))
 
 
-def bench_grid_update(torch, api, scene, steps, warmup, cell_order=False):
+def bench_grid_update(torch, api, scene, steps, warmup, cell_order=False, steady_state=False):
     w = scene.workload(5)
     s = api.OccupancySampler(w["sampler"])
     s.set_grid_sample_order(cell_order)
     s.init(1, w["resolution"], w["focal"], (0.5, 0.5), None, None, api.Pcg32(43))
     n_total = int(s.n_total_elements)
-    pos = torch.zeros((n_total, 3), device="cuda")
-    idx = torch.zeros(n_total, dtype=torch.int32, device="cuda")
+    # the reference's draw of its first 256 steps (one uniform point per cell) or of the steps after (a quarter each way)
+    n_uni, n_non = (n_total // 4, n_total // 4) if steady_state else (n_total, 0)
+    n_points = n_uni + n_non
+    pos = torch.zeros((n_points, 3), device="cuda")
+    idx = torch.zeros(n_points, dtype=torch.int32, device="cuda")
     g = torch.Generator(device="cuda")
     g.manual_seed(48)
-    dens = torch.nn.functional.softplus(torch.randn(n_total, generator=g, device="cuda")).half()
+    dens = torch.nn.functional.softplus(torch.randn(n_points, generator=g, device="cuda")).half()
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
     parts = {"sample_positions": [], "update_grid": [], "update_grid_bitfield": []}
 
     def step(record=False):
         if record:
             ev[0].record()
-        s.sample_positions_from_grid(n_total, 0, pos, idx)
+        s.sample_positions_from_grid(n_uni, n_non, pos, idx)
         if record:
             ev[1].record()
-        s.update_grid(n_total, 1, dens, idx, api.ACT_NONE)
+        s.update_grid(n_points, 1, dens, idx, api.ACT_NONE)
         if record:
             ev[2].record()
         s.update_grid_bitfield()
@@ -256,7 +259,8 @@ def bench_grid_update(torch, api, scene, steps, warmup, cell_order=False):
     avg = {k: sum(v) / len(v) for k, v in parts.items()}
     import numpy as np
     occ = float(np.unpackbits(s.density_grid_bitfield.cpu().numpy()).mean())
-    return dict(workload="grid_update_5" + ("_cell_order" if cell_order else ""), cells=n_total, ms_per_update=sec * 1e3, parts_ms=avg, occupied_bits=occ,
+    return dict(workload="grid_update_5" + ("_steady_state" if steady_state else "") + ("_cell_order" if cell_order else ""), cells=n_total, points=n_points,
+                ms_per_update=sec * 1e3, parts_ms=avg, occupied_bits=occ,
                 update_grid_gbs=EMA_BYTES_PER_CELL * n_total / (avg["update_grid"] * 1e-3) / 1e9,
                 bitfield_gbs=BITFIELD_BYTES_PER_CELL * n_total / (avg["update_grid_bitfield"] * 1e-3) / 1e9)
 
@@ -334,6 +338,8 @@ def main():
             torch.cuda.empty_cache()
         extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1))
         extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1, cell_order=True))
+        extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1, steady_state=True))
+        extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1, cell_order=True, steady_state=True))
         extras.append(bench_grid_sample_draws(torch, api, scene, max(2, args.steps // 2)))
         log(json.dumps(extras[-1]))
         out["extras"] = extras

@@ -160,9 +160,10 @@ int  srf_sampler_set_density_grid(srf_sampler_t* s, const float* density_grid, v
  * 0 (default): the reference's, point i in entry i.  1, cell order: with a power-of-two cell count n_cells (at least 2048) the
  * first n_cells * floor(n_uniform / n_cells) entries hold the same points sorted by the cell they fall in, entry
  * t = m * n_cells + v holding point i = ((v * A' - step * n_uniform) mod n_cells) + m * n_cells (A' the inverse of 56924617
- * modulo 2^32, step the number of srf_sampler_update_grid calls so far); every later entry is as in order 0.
- * srf_sampler_update_grid, given densities and indices in that same order, then combines those entries per cell without
- * sorting them (it checks each entry's index, so arrays in any other order still give the right grid, only slower).
+ * modulo 2^32, step the number of srf_sampler_update_grid calls so far); every later entry is as in order 0.  The non-uniform
+ * draw, whose entries follow those of the uniform one, is laid out the same way with n_nonuniform in place of n_uniform.
+ * srf_sampler_update_grid, given densities and indices in that same order, then combines the uniform draw's sorted entries per
+ * cell without sorting them (it checks each entry's index, so arrays in any other order still give the right grid, only slower).
  * The set of points, their positions and indices and the grid that results are those of order 0. */
 int  srf_sampler_set_grid_sample_order(srf_sampler_t* s, int32_t cell_order);
 

@@ -259,21 +259,27 @@ class OccupancySampler:
 
     def set_grid_sample_order(self, cell_order):
         """cell_order=True: sample_positions_from_grid leaves the uniform points of whole multiples of the cell count sorted by
-        cell (no counterpart in the reference; see grid_sample_entry_points for which point an entry holds) and update_grid,
-        given densities and indices in that order, splats them without sorting; the resulting grid is the same"""
+        cell, and likewise those of the non-uniform draw (no counterpart in the reference; see grid_sample_entry_points for
+        which point an entry holds); update_grid, given densities and indices in that order, splats the uniform ones without
+        sorting; the resulting grid is the same"""
         K.check(self._L.srf_sampler_set_grid_sample_order(self._h, 1 if cell_order else 0))
 
-    def grid_sample_entry_points(self, n_uniform, step=None):
-        """which point of the reference's order each of the first n_cells * (n_uniform // n_cells) entries holds in cell order
-        (numpy uint32 array); step: the number of update_grid calls before the draw (default: so far)"""
+    def grid_sample_entry_points(self, n_uniform, n_nonuniform=0, step=None):
+        """which point of the reference's order (uniform draw, then non-uniform draw) each entry of sample_positions_from_grid's
+        outputs holds in cell order (numpy int64 array of n_uniform + n_nonuniform entries); step: the number of update_grid
+        calls before the draw (default: so far)"""
         import numpy as np
         nc = int(self.info.n_grid_elements)
-        n_dealt = n_uniform // nc * nc if nc >= 2048 and nc & (nc - 1) == 0 else 0
         step = self.i_step if step is None else int(step)
-        t = np.arange(n_dealt, dtype=np.uint64)
         inv = pow(56924617, -1, 1 << 32)
-        u = ((t & (nc - 1)) * inv) & (nc - 1)
-        return (((u - step * n_uniform) & (nc - 1)) + (t // nc) * nc).astype(np.uint32)
+        parts = []
+        for first, n in ((0, int(n_uniform)), (int(n_uniform), int(n_nonuniform))):
+            n_dealt = n // nc * nc if nc >= 2048 and nc & (nc - 1) == 0 else 0
+            t = np.arange(n_dealt, dtype=np.int64)
+            u = ((t & (nc - 1)) * inv) & (nc - 1)
+            parts.append(first + ((u - step * n) & (nc - 1)) + (t // nc) * nc)
+            parts.append(first + np.arange(n_dealt, n, dtype=np.int64))
+        return np.concatenate(parts)
 
     def set_density_grid(self, grid):
         K.check(self._L.srf_sampler_set_density_grid(self._h, _dev(grid, torch.float32, self.info.n_total_elements, "grid"), _stream()))

@@ -72,11 +72,11 @@ __global__ void __launch_bounds__(256) k_generate_grid_samples_by_cell(Params P,
                                                                         const float* __restrict__ grid_in, float thresh,
                                                                         Float4* __restrict__ staged, const uint32_t* __restrict__ above,
                                                                         uint32_t tries_at_once, uint32_t a_inverse, uint32_t log2_cells,
-                                                                        float* __restrict__ positions, uint32_t* __restrict__ indices) {
+                                                                        float* __restrict__ positions, uint32_t* __restrict__ indices, uint32_t first_thread) {
 	__shared__ uint64_t skip_m[128], skip_p[128];
 	if (threadIdx.x < 128) pcg_skip16_entry(rng, threadIdx.x, &skip_m[threadIdx.x], &skip_p[threadIdx.x]);
 	__syncthreads();
-	const uint64_t t = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+	const uint64_t t = (uint64_t)first_thread + (uint64_t)blockIdx.x * 256u + threadIdx.x;      // staged holds the threads from first_thread on
 	const uint32_t mask = P.n_cells - 1u;
 	const uint32_t v = (uint32_t)t & mask, m = (uint32_t)(t >> log2_cells);
 	const uint32_t u = (v * a_inverse) & mask;                      // (i + step n) mod n_cells
@@ -86,17 +86,19 @@ __global__ void __launch_bounds__(256) k_generate_grid_samples_by_cell(Params P,
 	uint32_t idx;
 	grid_sample_point((uint32_t)i, P, n_elements, rng, step, grid_in, thresh, &pos, &idx, above, nullptr, tries_at_once, skip_m, skip_p);
 	// staged == NULL: the caller takes the points in this order (entry t of its arrays is thread t's point)
-	if (staged) staged[t] = mk4(pos.x, pos.y, pos.z, srf_u2f(idx));
+	if (staged) staged[t - first_thread] = mk4(pos.x, pos.y, pos.z, srf_u2f(idx));
 	else { st3(positions + 3 * (size_t)t, pos); indices[t] = idx; }
 }
 
 __global__ void __launch_bounds__(256) k_grid_samples_to_point_order(uint32_t n_cells, uint32_t n_elements, uint32_t step, uint32_t log2_cells,
-                                                                      const Float4* __restrict__ staged, float* __restrict__ positions, uint32_t* __restrict__ indices) {
-	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+                                                                      const Float4* __restrict__ staged, float* __restrict__ positions, uint32_t* __restrict__ indices,
+                                                                      uint32_t first) {
+	// the points from `first` (a multiple of the cell count) on; staged holds the threads from `first` on
+	const uint32_t i = first + blockIdx.x * blockDim.x + threadIdx.x;
 	if (i >= n_elements) return;
 	const uint32_t mask = n_cells - 1u;
 	const uint32_t v = (((i + step * n_elements) & mask) * 56924617u) & mask;      // the inverse of the dealing above
-	const Float4 r = staged[((uint64_t)(i >> log2_cells) << log2_cells) + v];
+	const Float4 r = staged[((uint64_t)(i >> log2_cells) << log2_cells) - first + v];
 	st3(positions + 3 * (size_t)i, mk3(r.x, r.y, r.z));
 	indices[i] = srf_f2u(r.w);
 }
@@ -612,7 +614,13 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	if (s->force_sample_by_cell >= 0) by_cell = s->force_sample_by_cell != 0 && can_deal;
 	// workspace: the two bit tables, then the staging array of the dealt draw (reserved in one go: growing frees)
 	const size_t table_bytes = tabulate ? align_up((size_t)div_up(s->n_total, 32) * 4, 256) : 0;
-	const uint64_t dealt_threads = by_cell ? (uint64_t)div_up(n_nonuniform, nc) * nc : 0;
+	// Cell order (srf_sampler_set_grid_sample_order): the points of whole multiples of the cell count stay in the order of the
+	// dealing, entry t = m n_cells + v of a draw holding the point whose (i + step n) A mod n_cells is v; srf_sampler_update_grid
+	// then splats the uniform ones without sorting.  The other points of each draw follow in their own order.
+	const bool cell_order = s->grid_sample_cell_order && (nc & (nc - 1u)) == 0u && nc >= DEALT_CELLS;
+	const uint32_t n_dealt = cell_order ? n_uniform / nc * nc : 0u, n_dealt_b = cell_order ? n_nonuniform / nc * nc : 0u;
+	by_cell = by_cell && n_nonuniform > n_dealt_b;
+	const uint64_t dealt_threads = by_cell ? (uint64_t)div_up(n_nonuniform, nc) * nc - n_dealt_b : 0;       // those that go through the staging array
 	const int rc = s->ws.reserve(2 * table_bytes + dealt_threads * sizeof(Float4) + 256);
 	if (rc != SRF_OK) return rc;
 	const uint32_t* above_a = nullptr;
@@ -630,14 +638,10 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	while ((1u << log2_cells) < nc) ++log2_cells;
 	uint32_t inv = 56924617u;                                  // inverse of the hash multiplier modulo 2^32, by Newton's iteration
 	for (int k = 0; k < 5; ++k) inv *= 2u - 56924617u * inv;
-	// Cell order (srf_sampler_set_grid_sample_order): the uniform points of whole multiples of the cell count stay in the order
-	// of the dealing, entry t = m n_cells + v holding the point whose (i + step n) A mod n_cells is v; srf_sampler_update_grid
-	// then splats them without sorting.  The other points follow in their own order.
-	const uint32_t n_dealt = s->grid_sample_cell_order && (nc & (nc - 1u)) == 0u && nc >= DEALT_CELLS ? n_uniform / nc * nc : 0u;
 	s->dealt_entries = n_dealt;
 	if (n_dealt) {
 		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(n_dealt / 256u), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, -0.01f, (Float4*)nullptr, above_a, 1u, inv, log2_cells, grid_positions, grid_indices);
+		                   (const float*)s->density_grid, -0.01f, (Float4*)nullptr, above_a, 1u, inv, log2_cells, grid_positions, grid_indices, 0u);
 		SRF_LAUNCH_CHECK();
 	}
 	if (n_uniform > n_dealt) {
@@ -649,17 +653,23 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	pcg_advance(s->rng, 1ull << 32);
 	float* positions_b = grid_positions + 3 * (size_t)n_uniform;
 	uint32_t* indices_b = grid_indices + n_uniform;
+	if (n_dealt_b) {
+		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(n_dealt_b / 256u), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, (Float4*)nullptr, above_b, tries, inv, log2_cells, positions_b, indices_b, 0u);
+		SRF_LAUNCH_CHECK();
+	}
 	if (by_cell) {
 		Float4* staged = (Float4*)((char*)s->ws.ptr + 2 * table_bytes);
 		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3((uint32_t)(dealt_threads / 256u)), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, staged, above_b, tries, inv, log2_cells, (float*)nullptr, (uint32_t*)nullptr);
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, staged, above_b, tries, inv, log2_cells, (float*)nullptr, (uint32_t*)nullptr, n_dealt_b);
 		SRF_LAUNCH_CHECK();
-		hipLaunchKernelGGL(k_grid_samples_to_point_order, dim3(div_up(n_nonuniform, 256)), dim3(256), 0, st, nc, n_nonuniform, s->i_step, log2_cells,
-		                   (const Float4*)staged, positions_b, indices_b);
+		hipLaunchKernelGGL(k_grid_samples_to_point_order, dim3(div_up(n_nonuniform - n_dealt_b, 256)), dim3(256), 0, st, nc, n_nonuniform, s->i_step, log2_cells,
+		                   (const Float4*)staged, positions_b, indices_b, n_dealt_b);
 		SRF_LAUNCH_CHECK();
-	} else if (n_nonuniform) {
-		hipLaunchKernelGGL(k_generate_grid_samples, dim3(div_up(n_nonuniform, 256) < 16384u ? div_up(n_nonuniform, 256) : 16384u), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, positions_b, indices_b, above_b, tries, 0u);
+	} else if (n_nonuniform > n_dealt_b) {
+		const uint32_t runs = div_up(n_nonuniform - n_dealt_b, 256);
+		hipLaunchKernelGGL(k_generate_grid_samples, dim3(runs < 16384u ? runs : 16384u), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, positions_b, indices_b, above_b, tries, n_dealt_b);
 		SRF_LAUNCH_CHECK();
 	}
 	pcg_advance(s->rng, 1ull << 32);

@@ -124,8 +124,8 @@ def test_grid_maintenance(gpu, orc, N, C, large_batch_path, monkeypatch):
 # update_grid, given densities and indices in that order, leaves the grid the oracle gets from the reference's order.
 # Step 0: every point in cell order (a whole multiple of the cell count).  Step 1: a grid with masked cells, so that some
 # uniform points settle on a later try (their entries do not lie in the cell the order puts them in), two and a half
-# multiples plus a non-uniform draw (the entries that follow in the reference's order go through the splat of small or, forced,
-# of large batches).  Step 2: fewer points than cells (nothing is in cell order).  Step 3: arrays handed to update_grid in
+# multiples plus a non-uniform draw of one and a half (the entries that are not the uniform draw's sorted ones go through the
+# splat of small or, forced, of large batches).  Step 2: fewer points than cells (nothing is in cell order).  Step 3: arrays handed to update_grid in
 # the reference's order although the sampler drew them in cell order (every entry fails its check; the grid is still right).
 @pytest.mark.parametrize("large_batch_path", ["0", "1"])
 @pytest.mark.parametrize("N,C", [((64, 32, 32), 5), ((128, 128, 128), 2)])
@@ -133,6 +133,7 @@ def test_grid_samples_in_cell_order(gpu, orc, N, C, large_batch_path, monkeypatc
     torch = gpu
     monkeypatch.setenv("SRF_SPLAT_SORT", large_batch_path)
     monkeypatch.setenv("SRF_GRID_SAMPLE_BITS", large_batch_path)
+    monkeypatch.setenv("SRF_GRID_SAMPLE_BY_CELL", large_batch_path)      # how the non-uniform points past the last whole multiple are drawn
     from sphericalrf_amd import api
     cfg = dict(warping_type="ERP", aabb_scale=16, grid_size=N, num_cascades=C, grid_distribution_type="WarpedSpace_Exp", init_grid_with_mask=False,
                maximum_marching_steps=256, sampling_type="Disparity", near_distance=0.05, far_distance=10.0)
@@ -145,7 +146,7 @@ def test_grid_samples_in_cell_order(gpu, orc, N, C, large_batch_path, monkeypatc
     o_grid = np.zeros(p.n_total, np.float32)
     rng = np.random.default_rng(2)
     nc, n_total = int(s.n_grid_elements), p.n_total
-    for step, (n_uni, n_non) in enumerate([(n_total, 0), (2 * nc + nc // 2, nc // 2), (nc // 2, nc // 4), (nc, 100)]):
+    for step, (n_uni, n_non) in enumerate([(n_total, 0), (2 * nc + nc // 2, nc + nc // 2), (nc // 2, nc // 4), (nc, 100)]):
         if step == 1:
             o_grid[rng.random(n_total) < 0.15] = -1.0          # masked cells: a uniform point that draws one tries the next candidate
             s.set_density_grid(torch.from_numpy(o_grid).cuda())
@@ -153,10 +154,11 @@ def test_grid_samples_in_cell_order(gpu, orc, N, C, large_batch_path, monkeypatc
         pos = torch.zeros((n, 3), dtype=torch.float32, device="cuda")
         idx = torch.zeros(n, dtype=torch.int32, device="cuda")
         assert s.i_step == step
-        entry_point = s.grid_sample_entry_points(n_uni)
+        order = s.grid_sample_entry_points(n_uni, n_non)
         n_dealt = n_uni // nc * nc
-        assert entry_point.shape == (n_dealt,) and np.array_equal(np.sort(entry_point), np.arange(n_dealt, dtype=np.uint32))
-        order = np.concatenate([entry_point, np.arange(n_dealt, n, dtype=np.uint32)]).astype(np.int64)
+        assert np.array_equal(np.sort(order), np.arange(n)) and np.array_equal(order[n_dealt:n_uni], np.arange(n_dealt, n_uni))
+        assert (n_dealt == 0) == (step == 2) and np.any(order[:n_dealt] != np.arange(n_dealt)) == (n_dealt != 0)
+        assert (order[n_uni:] != np.arange(n_uni, n)).any() == (n_non >= nc)
         s.sample_positions_from_grid(n_uni, n_non, pos, idx)
         wp1, wi1 = orc.generate_grid_samples(p, n_uni, o_rng, step, o_grid, -0.01)
         orc.advance(o_rng)
