@@ -1127,6 +1127,40 @@ def test_full_size_frame_after_a_grid_update_is_the_same_with_and_without_the_em
     assert int(out["table"][1].sum().item()) > 4 * n
 
 
+def test_full_size_grid_update_in_cell_order(gpu):
+    """Workload 5's draw and update at full size with the points left in cell order: the entries are the other order's points
+    in the documented permutation, and with the same density for the same point both orders leave the same grid."""
+    torch = gpu
+    from sphericalrf_amd import api, scene
+    w = scene.workload(5)
+    out = {}
+    for cell_order in (False, True):
+        s = api.OccupancySampler(w["sampler"])
+        s.set_grid_sample_order(cell_order)
+        s.init(1, w["resolution"], w["focal"], (0.5, 0.5), None, None, api.Pcg32(43))
+        n, nc = int(s.n_total_elements), int(s.n_grid_elements)
+        grids = []
+        for step in range(2):                  # the second draw runs against the grid the first update left, at step 1
+            pos = torch.zeros((n, 3), device="cuda")
+            idx = torch.zeros(n, dtype=torch.int32, device="cuda")
+            s.sample_positions_from_grid(n, 0, pos, idx)
+            # a density that depends on the point only (its cell and its position inside it), with zeros among them
+            dens = ((((idx.long() & 0xffffffff) * 2654435761 >> 13) & 0x3ff).float() / 64 * (pos[:, 0] - pos[:, 1]).abs()).half()
+            s.update_grid(n, 1, dens, idx, api.ACT_NONE)
+            grids.append(s.density_grid.clone())
+            if step == 1:
+                out[cell_order] = (pos, idx, grids)
+        del s
+    t = torch.arange(n, device="cuda")
+    inv = pow(56924617, -1, 1 << 32)
+    u = ((t & (nc - 1)) * inv) & (nc - 1)
+    order = ((u - 1 * n) & (nc - 1)) + (t // nc) * nc          # step 1
+    assert torch.equal(out[True][1], out[False][1][order]) and torch.equal(out[True][0], out[False][0][order])
+    assert not torch.equal(out[True][1], out[False][1])
+    for a, b in zip(out[True][2], out[False][2]):
+        assert torch.equal(a, b) and float((a > 0).float().mean().item()) > 0.3
+
+
 def test_full_size_grid_update_invariants(gpu):
     """Workload 5's grid maintenance at full size (167,772,160 cells): after one update from a zero grid the decayed max
     equals the largest splatted value per cell; the threshold is the cascade-0 mean (far below min_optical_thickness); every coarser cascade contains the pooled bits of the finer one; the table never allows skipping from
