@@ -190,25 +190,38 @@ __global__ void __launch_bounds__(256) k_splat_dealt(uint32_t n_cells, uint32_t 
 	const uint32_t cell0 = blockIdx.x * DEALT_CELLS;
 	for (uint32_t j = threadIdx.x; j < n_cascades * DEALT_CELLS; j += 256u) tiles[j] = 0u;
 	__syncthreads();
+	constexpr uint32_t PER_THREAD = DEALT_CELLS / 256u;     // entries of one multiple a thread takes: all fetched before any is used
 	for (uint32_t m = 0; m < n_blocks_m; ++m) {
-		for (uint32_t k = threadIdx.x; k < DEALT_CELLS; k += 256u) {
-			const uint32_t cell = cell0 + k;
+		uint32_t idx[PER_THREAD];
+		float raw[PER_THREAD];
+		#pragma unroll
+		for (uint32_t q = 0; q < PER_THREAD; ++q) {
+			const uint32_t cell = cell0 + q * 256u + threadIdx.x;
 			const size_t t = ((size_t)m << log2_cells) + ((cell - DEALT_FIRST_CELL) & mask);
-			const uint32_t idx = indices[t];
-			const float sigma = act_density(net_load<HALF>(densities, t * width), act);
-			const uint32_t bits = srf_f2u(sigma * min_cone_stepsize);
+			idx[q] = indices[t];
+			raw[q] = net_load<HALF>(densities, t * width);
+		}
+		#pragma unroll
+		for (uint32_t q = 0; q < PER_THREAD; ++q) {
+			const uint32_t k = q * 256u + threadIdx.x;
+			const uint32_t bits = srf_f2u(act_density(raw[q], act) * min_cone_stepsize);
 			if (bits == 0u) continue;                        // cannot raise a cell
-			const uint32_t level = idx >> log2_cells;
-			if ((idx & mask) == cell && level < n_cascades) atomicMax(&tiles[level * DEALT_CELLS + k], bits);
-			else { const uint32_t at = atomicAdd(list_count, 1u); U2 e; e.x = idx; e.y = bits; list[at] = e; }
+			const uint32_t level = idx[q] >> log2_cells;
+			if ((idx[q] & mask) == cell0 + k && level < n_cascades) atomicMax(&tiles[level * DEALT_CELLS + k], bits);
+			else { const uint32_t at = atomicAdd(list_count, 1u); U2 e; e.x = idx[q]; e.y = bits; list[at] = e; }
 		}
 	}
 	__syncthreads();
-	for (uint32_t j = threadIdx.x; j < n_cascades * DEALT_CELLS; j += 256u) {
-		const size_t at = (size_t)(j / DEALT_CELLS) * n_cells + cell0 + (j % DEALT_CELLS);
-		uint32_t v = tiles[j];
-		if (MERGE) { const uint32_t old = grid_current_bits[at]; v = old > v ? old : v; }
-		grid_current_bits[at] = v;
+	for (uint32_t level = 0; level < n_cascades; ++level) {
+		uint32_t* out = grid_current_bits + (size_t)level * n_cells + cell0;
+		uint32_t old[PER_THREAD];
+		#pragma unroll
+		for (uint32_t q = 0; q < PER_THREAD; ++q) old[q] = MERGE ? out[q * 256u + threadIdx.x] : 0u;
+		#pragma unroll
+		for (uint32_t q = 0; q < PER_THREAD; ++q) {
+			const uint32_t v = tiles[level * DEALT_CELLS + q * 256u + threadIdx.x];
+			out[q * 256u + threadIdx.x] = old[q] > v ? old[q] : v;
+		}
 	}
 }
 __global__ void __launch_bounds__(256) k_splat_listed(const uint32_t* __restrict__ list_count, const U2* __restrict__ list, uint32_t n_total, uint32_t* __restrict__ grid_current_bits) {
