@@ -72,22 +72,26 @@ __global__ void __launch_bounds__(256) k_generate_grid_samples_by_cell(Params P,
                                                                         const float* __restrict__ grid_in, float thresh,
                                                                         Float4* __restrict__ staged, const uint32_t* __restrict__ above,
                                                                         uint32_t tries_at_once, uint32_t a_inverse, uint32_t log2_cells,
-                                                                        float* __restrict__ positions, uint32_t* __restrict__ indices, uint32_t first_thread) {
+                                                                        float* __restrict__ positions, uint32_t* __restrict__ indices, uint32_t first_thread,
+                                                                        uint32_t n_runs) {
 	__shared__ uint64_t skip_m[128], skip_p[128];
 	if (threadIdx.x < 128) pcg_skip16_entry(rng, threadIdx.x, &skip_m[threadIdx.x], &skip_p[threadIdx.x]);
 	__syncthreads();
-	const uint64_t t = (uint64_t)first_thread + (uint64_t)blockIdx.x * 256u + threadIdx.x;      // staged holds the threads from first_thread on
-	const uint32_t mask = P.n_cells - 1u;
-	const uint32_t v = (uint32_t)t & mask, m = (uint32_t)(t >> log2_cells);
-	const uint32_t u = (v * a_inverse) & mask;                      // (i + step n) mod n_cells
-	const uint64_t i = (uint64_t)((u - step * n_elements) & mask) + ((uint64_t)m << log2_cells);
-	if (i >= n_elements) return;
-	Vec3 pos;
-	uint32_t idx;
-	grid_sample_point((uint32_t)i, P, n_elements, rng, step, grid_in, thresh, &pos, &idx, above, nullptr, tries_at_once, skip_m, skip_p);
-	// staged == NULL: the caller takes the points in this order (entry t of its arrays is thread t's point)
-	if (staged) staged[t - first_thread] = mk4(pos.x, pos.y, pos.z, srf_u2f(idx));
-	else { st3(positions + 3 * (size_t)t, pos); indices[t] = idx; }
+	// a workgroup takes several runs of 256 threads, so that the tables above are worked out a few thousand times, not once per run
+	for (uint32_t run = blockIdx.x; run < n_runs; run += gridDim.x) {
+		const uint64_t t = (uint64_t)first_thread + (uint64_t)run * 256u + threadIdx.x;      // staged holds the threads from first_thread on
+		const uint32_t mask = P.n_cells - 1u;
+		const uint32_t v = (uint32_t)t & mask, m = (uint32_t)(t >> log2_cells);
+		const uint32_t u = (v * a_inverse) & mask;                      // (i + step n) mod n_cells
+		const uint64_t i = (uint64_t)((u - step * n_elements) & mask) + ((uint64_t)m << log2_cells);
+		if (i >= n_elements) continue;
+		Vec3 pos;
+		uint32_t idx;
+		grid_sample_point((uint32_t)i, P, n_elements, rng, step, grid_in, thresh, &pos, &idx, above, nullptr, tries_at_once, skip_m, skip_p);
+		// staged == NULL: the caller takes the points in this order (entry t of its arrays is thread t's point)
+		if (staged) staged[t - first_thread] = mk4(pos.x, pos.y, pos.z, srf_u2f(idx));
+		else { st3(positions + 3 * (size_t)t, pos); indices[t] = idx; }
+	}
 }
 
 __global__ void __launch_bounds__(256) k_grid_samples_to_point_order(uint32_t n_cells, uint32_t n_elements, uint32_t step, uint32_t log2_cells,
@@ -647,14 +651,15 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 		above_a = a; above_b = b;
 	}
 	const uint32_t tries = 1;     // looking several candidates up at once (up to 4) has made no measurable difference
+	auto dealt_grid = [](uint32_t runs) { return runs < 16384u ? runs : 16384u; };
 	uint32_t log2_cells = 0;
 	while ((1u << log2_cells) < nc) ++log2_cells;
 	uint32_t inv = 56924617u;                                  // inverse of the hash multiplier modulo 2^32, by Newton's iteration
 	for (int k = 0; k < 5; ++k) inv *= 2u - 56924617u * inv;
 	s->dealt_entries = n_dealt;
 	if (n_dealt) {
-		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(n_dealt / 256u), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, -0.01f, (Float4*)nullptr, above_a, 1u, inv, log2_cells, grid_positions, grid_indices, 0u);
+		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(dealt_grid(n_dealt / 256u)), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, -0.01f, (Float4*)nullptr, above_a, 1u, inv, log2_cells, grid_positions, grid_indices, 0u, n_dealt / 256u);
 		SRF_LAUNCH_CHECK();
 	}
 	if (n_uniform > n_dealt) {
@@ -667,14 +672,15 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	float* positions_b = grid_positions + 3 * (size_t)n_uniform;
 	uint32_t* indices_b = grid_indices + n_uniform;
 	if (n_dealt_b) {
-		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(n_dealt_b / 256u), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, (Float4*)nullptr, above_b, tries, inv, log2_cells, positions_b, indices_b, 0u);
+		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(dealt_grid(n_dealt_b / 256u)), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, (Float4*)nullptr, above_b, tries, inv, log2_cells, positions_b, indices_b, 0u, n_dealt_b / 256u);
 		SRF_LAUNCH_CHECK();
 	}
 	if (by_cell) {
 		Float4* staged = (Float4*)((char*)s->ws.ptr + 2 * table_bytes);
-		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3((uint32_t)(dealt_threads / 256u)), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, staged, above_b, tries, inv, log2_cells, (float*)nullptr, (uint32_t*)nullptr, n_dealt_b);
+		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(dealt_grid((uint32_t)(dealt_threads / 256u))), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, staged, above_b, tries, inv, log2_cells, (float*)nullptr, (uint32_t*)nullptr, n_dealt_b,
+		                   (uint32_t)(dealt_threads / 256u));
 		SRF_LAUNCH_CHECK();
 		hipLaunchKernelGGL(k_grid_samples_to_point_order, dim3(div_up(n_nonuniform - n_dealt_b, 256)), dim3(256), 0, st, nc, n_nonuniform, s->i_step, log2_cells,
 		                   (const Float4*)staged, positions_b, indices_b, n_dealt_b);
