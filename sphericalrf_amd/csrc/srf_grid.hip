@@ -68,29 +68,56 @@ __global__ void __launch_bounds__(256) k_generate_grid_samples(Params P, uint32_
 // takes the m-th point with that v; which thread draws a point changes nothing in what is drawn.  The results go to a
 // staging array in thread order (16 bytes each, contiguous per wavefront); k_grid_samples_to_point_order then has thread i
 // fetch point i's record and write the outputs in their own order, so that neither kernel scatters its stores.
+constexpr uint32_t DEAL_WINDOW_MAX = 1024;      // threads of a window of k_generate_grid_samples_by_cell, at most
+// SPARSE: the launch covers a multiple of the cell count that the draw's points do not fill
+template <bool SPARSE>
 __global__ void __launch_bounds__(256) k_generate_grid_samples_by_cell(Params P, uint32_t n_elements, Pcg32 rng, uint32_t step,
                                                                         const float* __restrict__ grid_in, float thresh,
                                                                         Float4* __restrict__ staged, const uint32_t* __restrict__ above,
                                                                         uint32_t tries_at_once, uint32_t a_inverse, uint32_t log2_cells,
                                                                         float* __restrict__ positions, uint32_t* __restrict__ indices, uint32_t first_thread,
-                                                                        uint32_t n_runs) {
+                                                                        uint32_t n_windows, uint32_t per) {
 	__shared__ uint64_t skip_m[128], skip_p[128];
 	if (threadIdx.x < 128) pcg_skip16_entry(rng, threadIdx.x, &skip_m[threadIdx.x], &skip_p[threadIdx.x]);
 	__syncthreads();
-	// a workgroup takes several runs of 256 threads, so that the tables above are worked out a few thousand times, not once per run
-	for (uint32_t run = blockIdx.x; run < n_runs; run += gridDim.x) {
-		const uint64_t t = (uint64_t)first_thread + (uint64_t)run * 256u + threadIdx.x;      // staged holds the threads from first_thread on
-		const uint32_t mask = P.n_cells - 1u;
+	// A workgroup takes several windows of `per` x 256 threads (so that the tables above are worked out a few thousand times, not
+	// once per 256 points).  In a multiple of the cell count that the points do not fill only some of the threads have a point,
+	// scattered evenly over it: the window's threads that have one are listed first, and the workgroup's lanes then take the listed
+	// ones side by side.
+	__shared__ uint16_t live[DEAL_WINDOW_MAX];
+	__shared__ uint32_t n_live;
+	if (threadIdx.x == 0) n_live = 0u;
+	__syncthreads();
+	const uint32_t mask = P.n_cells - 1u;
+	auto point_of = [&](uint64_t t) -> uint64_t {
 		const uint32_t v = (uint32_t)t & mask, m = (uint32_t)(t >> log2_cells);
 		const uint32_t u = (v * a_inverse) & mask;                      // (i + step n) mod n_cells
-		const uint64_t i = (uint64_t)((u - step * n_elements) & mask) + ((uint64_t)m << log2_cells);
-		if (i >= n_elements) continue;
+		return (uint64_t)((u - step * n_elements) & mask) + ((uint64_t)m << log2_cells);
+	};
+	auto draw = [&](uint64_t t) {
 		Vec3 pos;
 		uint32_t idx;
-		grid_sample_point((uint32_t)i, P, n_elements, rng, step, grid_in, thresh, &pos, &idx, above, nullptr, tries_at_once, skip_m, skip_p);
+		grid_sample_point((uint32_t)point_of(t), P, n_elements, rng, step, grid_in, thresh, &pos, &idx, above, nullptr, tries_at_once, skip_m, skip_p);
 		// staged == NULL: the caller takes the points in this order (entry t of its arrays is thread t's point)
 		if (staged) staged[t - first_thread] = mk4(pos.x, pos.y, pos.z, srf_u2f(idx));
 		else { st3(positions + 3 * (size_t)t, pos); indices[t] = idx; }
+	};
+	for (uint32_t win = blockIdx.x; win < n_windows; win += gridDim.x) {
+		const uint64_t t0 = (uint64_t)first_thread + (uint64_t)win * (per * 256u);      // staged holds the threads from first_thread on
+		if (!SPARSE) {                       // every thread has a point
+			for (uint32_t q = 0; q < per; ++q) draw(t0 + q * 256u + threadIdx.x);
+			continue;
+		}
+		uint32_t mine = 0, count = 0;
+		for (uint32_t q = 0; q < per; ++q) if (point_of(t0 + q * 256u + threadIdx.x) < n_elements) { mine |= 1u << q; ++count; }
+		uint32_t slot = count ? atomicAdd(&n_live, count) : 0u;
+		for (uint32_t q = 0; q < per; ++q) if (mine >> q & 1u) live[slot++] = (uint16_t)(q * 256u + threadIdx.x);
+		__syncthreads();
+		const uint32_t n = n_live;
+		for (uint32_t k = threadIdx.x; k < n; k += 256u) draw(t0 + live[k]);
+		__syncthreads();
+		if (threadIdx.x == 0) n_live = 0u;
+		__syncthreads();
 	}
 }
 
@@ -651,15 +678,16 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 		above_a = a; above_b = b;
 	}
 	const uint32_t tries = 1;     // looking several candidates up at once (up to 4) has made no measurable difference
-	auto dealt_grid = [](uint32_t runs) { return runs < 16384u ? runs : 16384u; };
+	auto dealt_grid = [](uint32_t windows) { return windows < 16384u ? windows : 16384u; };
+	const uint32_t deal_window = nc >= DEAL_WINDOW_MAX ? DEAL_WINDOW_MAX : 256u;      // threads of the dealing a workgroup takes at a time (the cell count, a power of two >= 256, is a multiple)
 	uint32_t log2_cells = 0;
 	while ((1u << log2_cells) < nc) ++log2_cells;
 	uint32_t inv = 56924617u;                                  // inverse of the hash multiplier modulo 2^32, by Newton's iteration
 	for (int k = 0; k < 5; ++k) inv *= 2u - 56924617u * inv;
 	s->dealt_entries = n_dealt;
 	if (n_dealt) {
-		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(dealt_grid(n_dealt / 256u)), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, -0.01f, (Float4*)nullptr, above_a, 1u, inv, log2_cells, grid_positions, grid_indices, 0u, n_dealt / 256u);
+		hipLaunchKernelGGL(k_generate_grid_samples_by_cell<false>, dim3(dealt_grid(n_dealt / deal_window)), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, -0.01f, (Float4*)nullptr, above_a, 1u, inv, log2_cells, grid_positions, grid_indices, 0u, n_dealt / deal_window, deal_window / 256u);
 		SRF_LAUNCH_CHECK();
 	}
 	if (n_uniform > n_dealt) {
@@ -672,16 +700,26 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	float* positions_b = grid_positions + 3 * (size_t)n_uniform;
 	uint32_t* indices_b = grid_indices + n_uniform;
 	if (n_dealt_b) {
-		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(dealt_grid(n_dealt_b / 256u)), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, (Float4*)nullptr, above_b, tries, inv, log2_cells, positions_b, indices_b, 0u, n_dealt_b / 256u);
+		hipLaunchKernelGGL(k_generate_grid_samples_by_cell<false>, dim3(dealt_grid(n_dealt_b / deal_window)), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, (Float4*)nullptr, above_b, tries, inv, log2_cells, positions_b, indices_b, 0u, n_dealt_b / deal_window, deal_window / 256u);
 		SRF_LAUNCH_CHECK();
 	}
 	if (by_cell) {
 		Float4* staged = (Float4*)((char*)s->ws.ptr + 2 * table_bytes);
-		hipLaunchKernelGGL(k_generate_grid_samples_by_cell, dim3(dealt_grid((uint32_t)(dealt_threads / 256u))), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, staged, above_b, tries, inv, log2_cells, (float*)nullptr, (uint32_t*)nullptr, n_dealt_b,
-		                   (uint32_t)(dealt_threads / 256u));
-		SRF_LAUNCH_CHECK();
+		// the whole multiples of the cell count, then the one the points do not fill
+		const uint64_t full_threads = (uint64_t)n_nonuniform / nc * nc - n_dealt_b;
+		if (full_threads) {
+			hipLaunchKernelGGL(k_generate_grid_samples_by_cell<false>, dim3(dealt_grid((uint32_t)(full_threads / deal_window))), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
+			                   (const float*)s->density_grid, s->P.min_optical_thickness, staged, above_b, tries, inv, log2_cells, (float*)nullptr, (uint32_t*)nullptr, n_dealt_b,
+			                   (uint32_t)(full_threads / deal_window), deal_window / 256u);
+			SRF_LAUNCH_CHECK();
+		}
+		if (dealt_threads > full_threads) {
+			hipLaunchKernelGGL(k_generate_grid_samples_by_cell<true>, dim3(dealt_grid(nc / deal_window)), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
+			                   (const float*)s->density_grid, s->P.min_optical_thickness, staged + full_threads, above_b, tries, inv, log2_cells, (float*)nullptr, (uint32_t*)nullptr,
+			                   (uint32_t)(n_dealt_b + full_threads), nc / deal_window, deal_window / 256u);
+			SRF_LAUNCH_CHECK();
+		}
 		hipLaunchKernelGGL(k_grid_samples_to_point_order, dim3(div_up(n_nonuniform - n_dealt_b, 256)), dim3(256), 0, st, nc, n_nonuniform, s->i_step, log2_cells,
 		                   (const Float4*)staged, positions_b, indices_b, n_dealt_b);
 		SRF_LAUNCH_CHECK();
