@@ -211,6 +211,7 @@ __global__ void __launch_bounds__(256) k_splat_slabs(uint32_t n_elements, uint32
 // elsewhere (a later try, or arrays that are not in this order at all) goes to a list that k_splat_listed applies afterwards.
 // MERGE: the cells already hold the splat of other samples (those not in this order), so the result is the larger of both.
 constexpr uint32_t DEALT_CELLS = 2048;
+constexpr uint32_t DEALT_MAX_CASCADES = 8;            // 64 KB of LDS a workgroup; grids of more cascades take the entries through the other paths
 constexpr uint32_t DEALT_FIRST_CELL = 96925573u;      // the constant of the candidate-cell hash (grid_sample_tries)
 template <bool HALF, bool MERGE>
 __global__ void __launch_bounds__(256) k_splat_dealt(uint32_t n_cells, uint32_t log2_cells, uint32_t n_cascades, uint32_t n_blocks_m, const uint32_t* __restrict__ indices,
@@ -748,7 +749,7 @@ int srf_sampler_update_grid(srf_sampler_t* s, uint32_t n_total_positions, uint32
 	// the leading entries that the last srf_sampler_sample_positions_from_grid left in cell order (every one of them is checked
 	// where it is used: arrays in another order cost time, not correctness), and the others
 	uint32_t n_dealt = s->grid_sample_cell_order && s->dealt_entries < n_total_positions ? s->dealt_entries : (s->grid_sample_cell_order ? n_total_positions : 0u);
-	n_dealt = (nc & (nc - 1u)) == 0u && nc >= DEALT_CELLS ? n_dealt / nc * nc : 0u;
+	n_dealt = (nc & (nc - 1u)) == 0u && nc >= DEALT_CELLS && s->P.n_cascades <= DEALT_MAX_CASCADES ? n_dealt / nc * nc : 0u;
 	const uint32_t n = n_total_positions - n_dealt;
 	const uint32_t* rest_indices = grid_indices ? grid_indices + n_dealt : nullptr;
 	const void* rest_densities = grid_densities ? (const char*)grid_densities + (size_t)n_dealt * padded_output_width * (half ? 2 : 4) : nullptr;
