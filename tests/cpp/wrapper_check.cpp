@@ -28,6 +28,8 @@ int main() {
 		if (m.n_grid_elements != 32u * 16u * 16u || m.n_cascades != 3 || m.n_total_elements != 3u * 32u * 16u * 16u) return 1;
 		if (!(m.min_cone_stepsize > 0.f) || m.aabb_min[0] != 0.5f - 8.f || m.aabb_max[2] != 0.5f + 8.f) return 1;
 		sampler.update_grid_bitfield(nullptr);
+		sampler.set_grid_sample_order(true);
+		sampler.set_grid_sample_order(false);
 		srf::RayMarcher marcher(srf::RayMarcher::default_config());
 		marcher.sync_check(nullptr);
 		if (marcher.config().transmittance_threshold <= 0.f) return 1;
