@@ -160,34 +160,45 @@ SRF_HD bool mask_camera_sees(const float* m, Vec3 p, float radius, float focal_x
 // hashed cells for one above the threshold, jitter a point inside it.
 // ------------------------------------------------------------------------------------
 // occupancy_sampler.cu:121-130 — the up to ten tries of one point; POW2: the cell count is a power of two
-template <bool POW2>
-SRF_HD void grid_sample_tries(uint32_t i, const Params& P, uint32_t n_elements, uint32_t step, uint32_t level, const float* grid_in, float thresh,
-                              const uint32_t* above, uint32_t tries_at_once, uint32_t* cell_out, uint32_t* idx_out) {
-	// The ten candidate cells do not depend on what the grid holds, so several can be looked up side by side
-	// (tries_at_once, at most 4); the first that passes, in the reference's order, is taken, the tenth if none does.
-	// One dependent lookup after the other makes a wavefront wait for its unluckiest lane, a memory round trip per try.
+// The ten candidate cells do not depend on what the grid holds, so BATCH of them (1, 2, 5 or 10) are looked up side by side;
+// the first that passes, in the reference's order, is taken, the tenth if none does.  One dependent lookup after the other
+// makes a wavefront wait for its unluckiest lane, a memory round trip per try.
+template <bool POW2, uint32_t BATCH>
+SRF_HD void grid_sample_tries_batched(uint32_t i, const Params& P, uint32_t n_elements, uint32_t step, uint32_t level, const float* grid_in, float thresh,
+                                      const uint32_t* above, uint32_t* cell_out, uint32_t* idx_out) {
+	static_assert(10 % BATCH == 0, "whole batches");
 	uint32_t cell = 0, idx = 0;
 	bool found = false;
-	const uint32_t batch = tries_at_once < 1u ? 1u : (tries_at_once > 4u ? 4u : tries_at_once);
-	for (uint32_t j0 = 0; j0 < 10 && !found; j0 += batch) {
-		uint32_t c[4], id[4];
-		bool pass[4];
-		for (uint32_t q = 0; q < 4; ++q) {
-			const uint32_t j = j0 + q;
-			pass[q] = false; c[q] = 0; id[q] = 0;
-			if (q < batch && j < 10) {
-				const uint32_t h = (i + step * n_elements) * 56924617u + j * 19349663u + 96925573u;
-				c[q] = POW2 ? (h & (P.n_cells - 1u)) : (h % P.n_cells);
-				id[q] = c[q] + level * P.n_cells;
-				pass[q] = above ? ((above[id[q] >> 5] >> (id[q] & 31u)) & 1u) != 0u : grid_in[id[q]] > thresh;
-			}
+	const uint32_t h0 = (i + step * n_elements) * 56924617u + 96925573u;
+	for (uint32_t j0 = 0; j0 < 10 && !found; j0 += BATCH) {
+		uint32_t c[BATCH], id[BATCH];
+		bool pass[BATCH];
+#if defined(__HIP_DEVICE_COMPILE__)
+		#pragma unroll
+#endif
+		for (uint32_t q = 0; q < BATCH; ++q) {
+			const uint32_t h = h0 + (j0 + q) * 19349663u;
+			c[q] = POW2 ? (h & (P.n_cells - 1u)) : (h % P.n_cells);
+			id[q] = c[q] + level * P.n_cells;
+			pass[q] = above ? ((above[id[q] >> 5] >> (id[q] & 31u)) & 1u) != 0u : grid_in[id[q]] > thresh;
 		}
-		for (uint32_t q = 0; q < 4 && !found; ++q) {
-			if (q < batch && j0 + q < 10) { cell = c[q]; idx = id[q]; found = pass[q]; }
+#if defined(__HIP_DEVICE_COMPILE__)
+		#pragma unroll
+#endif
+		for (uint32_t q = 0; q < BATCH; ++q) {
+			if (!found) { cell = c[q]; idx = id[q]; found = pass[q]; }
 		}
 	}
 	*cell_out = cell;
 	*idx_out = idx;
+}
+template <bool POW2>
+SRF_HD void grid_sample_tries(uint32_t i, const Params& P, uint32_t n_elements, uint32_t step, uint32_t level, const float* grid_in, float thresh,
+                              const uint32_t* above, uint32_t tries_at_once, uint32_t* cell_out, uint32_t* idx_out) {
+	if (tries_at_once >= 10u) grid_sample_tries_batched<POW2, 10>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out);
+	else if (tries_at_once >= 5u) grid_sample_tries_batched<POW2, 5>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out);
+	else if (tries_at_once >= 2u) grid_sample_tries_batched<POW2, 2>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out);
+	else grid_sample_tries_batched<POW2, 1>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out);
 }
 
 // above: optional table of the comparison grid_in[idx] > thresh, one bit per cell (bit idx & 31 of word idx >> 5),
