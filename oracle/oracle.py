@@ -113,11 +113,13 @@ def _f3(x):
 class Oracle:
     """One loaded oracle library (shared-definition build by default, glibc build with libm=True)."""
 
-    def __init__(self, libm=False):
-        name = "liboracle_libm.so" if libm else "liboracle.so"
-        path = os.path.join(_HERE, name)
-        if not os.path.exists(path):
-            build()
+    def __init__(self, libm=False, path=None):
+        """path: a library built elsewhere from a (deliberately altered) copy of srf_oracle.cpp; the mutation tests use it"""
+        if path is None:
+            name = "liboracle_libm.so" if libm else "liboracle.so"
+            path = os.path.join(_HERE, name)
+            if not os.path.exists(path):
+                build()
         self.lib = L = C.CDLL(path)
         L.orc_max_threads.restype = C.c_int
         L.orc_uses_libm.restype = C.c_int
