@@ -8,7 +8,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIBDIR = os.path.join(_HERE, "lib")
 LIB = os.path.join(LIBDIR, "libsrf_hip.so")
-SOURCES = ["srf_common.hip", "srf_grid.hip", "srf_march.hip", "srf_composite.hip", "srf_frame.hip"]
+SOURCES = ["srf_common.hip", "srf_grid.hip", "srf_march.hip", "srf_composite.hip", "srf_composite_waves.hip", "srf_frame.hip"]
 
 # -ffp-contract=off: a*b+c stays two rounded operations so host and device agree bit for bit.
 # packed-fp32-ops is switched off because some packed forms have produced wrong results on this hardware.
@@ -38,7 +38,7 @@ def _compile(src, extra):
 
 def build(verbose=False, extra_flags=()):
     os.makedirs(LIBDIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=6) as ex:
         results = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
     objs = [o for o, _ in results]
     if verbose:

@@ -72,6 +72,7 @@ struct srf_sampler {
 struct srf_marcher {
 	srf_marcher_config cfg;
 	srf::Workspace ws;          // ordered-offset chain of the streaming compositing kernel
+	srf::Workspace wave_ws;     // ordered-offset chain and item table of the wave-per-item compositing kernel
 	srf::Workspace ws2;         // per-ray forward results of the three-launch compositing
 	srf::Workspace reg;         // reg_distortion_buffer (ray_marcher.h:79-80)
 	srf::Workspace compact_ws;  // per-block counts of srf_compact_rays
@@ -80,6 +81,7 @@ struct srf_marcher {
 	unsigned long long* frame_word_dev = nullptr;   // device address of the second of them (8 bytes in), which the compaction kernel writes itself
 	uint32_t frame_stamp = 0;                // number of the last compaction srf_render_frame waited for
 	bool force_unfused = false;             // SRF_COMPOSITE_IMPL=unfused at creation
+	bool force_stream = false;              // SRF_COMPOSITE_IMPL=stream at creation
 	bool degraded = false;                  // the chain has failed once: every later call uses the three-launch implementation
 	volatile uint32_t* host_error = nullptr; // host word the streaming kernel raises when its chain gives up (pinned, device-writable)
 	uint32_t* host_error_dev = nullptr;      // the same word as the device addresses it
@@ -88,6 +90,14 @@ struct srf_marcher {
 };
 
 namespace srf {
+struct LossConst;
+// the wave-per-item training compositing (srf_composite_waves.hip): device scratch it needs for a call of n_rays rays (the first 512
+// bytes zero before the first call, and left zero by every call), where its error word lies, and the two launches
+size_t waves_scratch_bytes(uint32_t n_rays);
+uint32_t* waves_error_word(void* scratch);
+int launch_waves(const srf_loss_args* a, const LossConst& K, void* scratch, uint32_t* host_error, uint32_t spin_limit, const float* rays_rgba, const uint32_t* n_rays_counter,
+                 uint32_t* ray_coord_indices, const float* dt, const float* coords, float* compacted_coords, uint32_t* n_compacted_coords_counter,
+                 const void* network_output, void* dloss_doutput, float* loss_output, const float* density_grid_mean, float* rgb_ray_out, hipStream_t st);
 // srf_compact_rays with two more choices: alive_from_zero numbers the live rays from 0 whatever *n_alive_counter holds; host_word
 // (device address of a word of host memory, or NULL) receives stamp << 32 | the live-ray counter's new value when the call is done
 int compact_rays(srf_marcher* m, uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba,

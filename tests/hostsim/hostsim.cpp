@@ -13,6 +13,7 @@ static uint64_t g_radius_hist[8][4] = {};   // [cascade][radius 0, 1-block, 2-3,
 #include <algorithm>
 #include "../../sphericalrf_amd/csrc/srf_bodies.h"
 #include "../../sphericalrf_amd/csrc/srf_composite_fused.h"
+#include "../../sphericalrf_amd/csrc/srf_composite_wave.h"
 #include "../../oracle/srf_oracle.h"
 
 using namespace srf;
@@ -182,6 +183,136 @@ static void run_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n
 	*n_compacted_counter = prefix;
 	slow_groups(true);
 	delete[] ws; delete ww; delete rlp;
+}
+
+// The wave-per-item compositing, item by item and phase by phase, in the control flow of the device kernel: the
+// preparing pass (stride of the sample windows, first ray of every item, whether the rays are laid out in order),
+// then every item in order.  An item's rays go through the LDS window 64 at a time (a batch): a batch whose samples
+// fit the window in one piece, or chunk by chunk with a second sweep for the gradients; an item of several batches
+// counts all of them first.  Every item of a call whose rays are not in order is composited one lane per ray from memory.
+// counts: batches that fit the window / chunked batches / per-ray items / items of several batches.
+template <bool HI, bool HO>
+static void run_wave(const orc_loss_args* a, const float* rays_rgba, uint32_t n_rays_counter, uint32_t* ray_coord_indices, const float* dt,
+                     const float* coords, float* compacted_coords, uint32_t* n_compacted_counter, const void* net, void* dloss, float* loss_output,
+                     float* rgb_ray_out, uint32_t counts[4], uint32_t force_stride) {
+	using namespace wv;
+	Args A;
+	A.K = make_loss_const(a);
+	A.n_active = n_rays_counter < a->n_rays ? n_rays_counter : a->n_rays;
+	A.rays_rgba = rays_rgba; A.ray_coord_indices = ray_coord_indices; A.dt_arr = dt; A.coords = coords; A.compacted_coords = compacted_coords;
+	A.net = net; A.dloss = dloss; A.loss_output = loss_output; A.rgb_ray_out = rgb_ray_out; A.mean_density = a->mean_density;
+	const bool plain = A.K.rgb_act == SRF_ACT_NONE && A.K.density_act == SRF_ACT_NONE;
+	const uint32_t cap = max_items(a->n_rays);
+	// preparing pass
+	Windows W = windows_of(A.n_active, ray_coord_indices, cap);
+	if (force_stride) { W.stride = force_stride; W.n_items = A.n_active ? (uint32_t)((ray_coord_indices[2 * (size_t)(A.n_active - 1) + 1] - W.base0) / W.stride) + 1 : 0; }
+	std::vector<uint32_t> item_first((size_t)cap + 1, 0xdeadbeefu);
+	bool irregular = false;
+	for (uint32_t i = 0; i < A.n_active; ++i) if (!prepare_ray(i, A.n_active, ray_coord_indices, W, cap, item_first.data())) irregular = true;
+	if (!irregular && W.n_items > cap) irregular = true;      // (a forced stride may ask for more items than the table holds)
+	const uint32_t n_items = irregular ? (A.n_active + GROUP - 1) / GROUP : W.n_items;
+	Lds* wp = new Lds();
+	Lds& w = *wp;
+	std::vector<SlotState<G, HI>> st(LANES);
+	uint32_t prefix = *n_compacted_counter;
+
+	// one batch: rays [rb, rb + nb) of the call, nb <= 64
+	struct Batch { uint32_t rb, nb; uint64_t s0; uint32_t range, n_chunks; uint32_t n[LANES], rbase[LANES]; Float4 tgt[LANES]; RayState rs[LANES]; };
+	Batch B;
+	auto load_batch = [&](uint32_t rb, uint32_t nb) {
+		B.rb = rb; B.nb = nb;
+		uint64_t base[LANES];
+		for (uint32_t l = 0; l < LANES; ++l) {
+			B.n[l] = 0; base[l] = 0; B.tgt[l] = mk4(0.f, 0.f, 0.f, 0.f);
+			if (l < nb) { B.n[l] = ray_coord_indices[2 * (size_t)(rb + l)]; base[l] = ray_coord_indices[2 * (size_t)(rb + l) + 1]; B.tgt[l] = *(const Float4*)(rays_rgba + 4 * (size_t)(rb + l)); }
+		}
+		B.s0 = nb ? base[0] : 0;
+		B.range = nb ? (uint32_t)(base[nb - 1] + B.n[nb - 1] - B.s0) : 0;
+		for (uint32_t l = 0; l < LANES; ++l) B.rbase[l] = l < nb ? (uint32_t)(base[l] - B.s0) : B.range;
+		B.n_chunks = (B.range + WIN - 1) / WIN;
+	};
+	auto rows = [&](uint32_t chunk_lo) {
+		for (uint32_t l = 0; l < LANES; ++l) rows_load<HI>(l, A, B.s0, B.range, chunk_lo, st[l]);
+		for (uint32_t l = 0; l < LANES; ++l) { if (plain) rows_alpha<HI, true>(l, A, w, B.range, chunk_lo, st[l]); else rows_alpha<HI, false>(l, A, w, B.range, chunk_lo, st[l]); }
+	};
+	auto chain_all = [&](uint32_t chunk_lo) {
+		uint32_t steps = 0;
+		for (uint32_t l = 0; l < LANES; ++l) { uint32_t k0, k1; chain_span(B.n[l], B.rbase[l], chunk_lo, &k0, &k1); steps = k1 - k0 > steps ? k1 - k0 : steps; }
+		// stretch by stretch across the lanes, as the wavefront runs it (with its early exit)
+		for (uint32_t j = 0; j < steps; j += CHAIN_UNROLL) {
+			bool any_live = false;
+			for (uint32_t l = 0; l < LANES; ++l) { uint32_t k0, k1; chain_span(B.n[l], B.rbase[l], chunk_lo, &k0, &k1); if (k0 + j < k1 && B.rs[l].dead == 0) any_live = true; }
+			if (!any_live) break;
+			for (uint32_t l = 0; l < LANES; ++l) { uint32_t k0, k1; chain_span(B.n[l], B.rbase[l], chunk_lo, &k0, &k1); chain_stretch(l, j, k0, k1, B.rbase[l], chunk_lo, A.K.thr, w, B.rs[l]); }
+		}
+	};
+	auto grads = [&](uint32_t chunk_lo) {
+		for (uint32_t l = 0; l < LANES; ++l) {
+			if (plain) rows_grads<HI, HO, true>(l, A, w, B.s0, B.range, chunk_lo, st[l]); else rows_grads<HI, HO, false>(l, A, w, B.s0, B.range, chunk_lo, st[l]);
+		}
+	};
+	auto forward = [&]() {       // every chunk's rows and chain; the last chunk's records stay in the window
+		for (uint32_t l = 0; l < LANES; ++l) ray_reset(B.rs[l]);
+		for (uint32_t c = 0; c < (B.n_chunks ? B.n_chunks : 1u); ++c) { rows(c * WIN); chain_all(c * WIN); }
+	};
+	auto batch_total = [&]() { uint32_t t = 0; for (uint32_t l = 0; l < B.nb; ++l) t += B.rs[l].cnt; return t; };
+	auto finish_commit_grads = [&](uint32_t cbase0) {     // after forward(), with the batch's first compacted offset known
+		float loss[LANES];
+		for (uint32_t l = 0; l < B.nb; ++l) loss[l] = finish_lane(l, B.rb + l, B.n[l], A, w, B.rs[l], B.tgt[l]);
+		uint32_t run = cbase0;
+		for (uint32_t l = 0; l < LANES; ++l) {
+			if (l < B.nb) { commit_lane(l, B.rb + l, B.rs[l].cnt, B.rbase[l], run, loss[l], A, w); run += B.rs[l].cnt; } else commit_none(l, w);
+		}
+		if (B.n_chunks <= 1) { ++counts[0]; grads(0); }
+		else {
+			++counts[1];
+			for (uint32_t l = 0; l < LANES; ++l) ray_reset(B.rs[l]);
+			for (uint32_t c = 0; c < B.n_chunks; ++c) { rows(c * WIN); chain_all(c * WIN); grads(c * WIN); }
+		}
+	};
+
+	for (uint32_t item = 0; item < n_items; ++item) {
+		uint32_t r0, n_r;
+		if (irregular) { r0 = item * GROUP; n_r = A.n_active - r0 < GROUP ? A.n_active - r0 : GROUP; }
+		else { r0 = item_first[item]; n_r = item_first[item + 1] - r0; }
+		if (!irregular) {
+			const uint32_t n_batches = (n_r + LANES - 1) / LANES;
+			if (n_batches <= 1) {
+				load_batch(r0, n_r);
+				forward();
+				const uint32_t total = batch_total();
+				finish_commit_grads(prefix);        // (the device publishes the total and chains it to the earlier items' here)
+				prefix += total;
+			} else {
+				++counts[3];
+				uint32_t total = 0;
+				for (uint32_t b = 0; b < n_batches; ++b) { load_batch(r0 + b * LANES, n_r - b * LANES < LANES ? n_r - b * LANES : LANES); forward(); total += batch_total(); }
+				uint32_t run = prefix;
+				for (uint32_t b = 0; b < n_batches; ++b) {
+					load_batch(r0 + b * LANES, n_r - b * LANES < LANES ? n_r - b * LANES : LANES);
+					forward();
+					const uint32_t t = batch_total();
+					finish_commit_grads(run);
+					run += t;
+				}
+				prefix += total;
+			}
+		} else {
+			++counts[2];
+			std::vector<FwdRay> fw(n_r);
+			std::vector<uint32_t> nf(n_r, 0);
+			for (uint32_t k = 0; k < n_r; ++k) loss_forward_body<HI>(r0 + k, A.K, A.rays_rgba, A.n_active, A.ray_coord_indices, A.dt_arr, A.net, &fw[k], &nf[k], A.rgb_ray_out);
+			uint32_t run = prefix;
+			for (uint32_t k = 0; k < n_r; ++k) {
+				loss_backward_body<HI, HO>(r0 + k, A.K, A.n_active, A.ray_coord_indices, A.dt_arr, A.coords, A.compacted_coords, A.net, A.dloss, A.loss_output,
+				                           A.mean_density, fw[k], nf[k], run, nullptr);
+				run += nf[k];
+			}
+			prefix = run;
+		}
+	}
+	*n_compacted_counter = prefix;
+	delete wp;
 }
 
 extern "C" {
@@ -551,6 +682,18 @@ void hs_loss_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n_ra
 	if (hin && hout) RUN(true, true); else if (hin) RUN(true, false); else if (hout) RUN(false, true); else RUN(false, false);
 #undef RUN
 }
+
+void hs_loss_wave(const orc_loss_args* a, const float* rays_rgba, uint32_t n_rays_counter, uint32_t* ray_coord_indices, const float* dt,
+                  const float* coords, float* compacted_coords, uint32_t* n_compacted_counter, const void* net, void* dloss, float* loss_output,
+                  float* rgb_ray_out, uint32_t counts[4], uint32_t force_stride) {
+	const bool hin = a->network_output_dtype == ORC_DTYPE_F16, hout = a->dloss_dtype == ORC_DTYPE_F16;
+	counts[0] = counts[1] = counts[2] = counts[3] = 0;
+#define RUN(HI, HO) run_wave<HI, HO>(a, rays_rgba, n_rays_counter, ray_coord_indices, dt, coords, compacted_coords, n_compacted_counter, net, dloss, loss_output, rgb_ray_out, counts, force_stride)
+	if (hin && hout) RUN(true, true); else if (hin) RUN(true, false); else if (hout) RUN(false, true); else RUN(false, false);
+#undef RUN
+}
+
+uint32_t hs_window_stride(uint32_t n_active, uint64_t span, uint64_t end, uint32_t item_cap) { return wv::window_stride(n_active, span, end, item_cap); }
 
 
 void hs_volume_rendering(const orc_params* p, const orc_render_args* a, srf_ray_payload* payloads, float* rgba, const float* coords, const void* net) {

@@ -57,7 +57,7 @@ def test_fused_equals_oracle(orc, hostsim, kind, hin, hout):
               background_color=(O.f32 * 3)(0.1, 0.7, 0.3), mean_density=0.001)
     a = loss_args(n_rays, cap, **kw)
     outs = []
-    for fn in ("oracle", "fused"):
+    for fn in ("oracle", "fused", "wave", "wave_stride_128", "wave_stride_4096"):
         idx = np.stack([counts, base], axis=1).astype(np.uint32)
         dloss = np.zeros((cap, 4), np.float16 if hout else np.float32)
         comp = np.zeros((cap, 7), np.float32)
@@ -68,6 +68,26 @@ def test_fused_equals_oracle(orc, hostsim, kind, hin, hout):
         if fn == "oracle":
             tot = orc.volume_rendering_with_loss_and_gradient(a, tgt, n_active, idx, dt, net, dloss, n_compacted_counter=11, coords=coords,
                                                               compacted_coords=comp, loss_output=loss, rgb_ray_out=rgb)
+        elif fn.startswith("wave"):
+            # the wave-per-item kernel's control flow, with the stride of the sample windows it would choose and with two forced ones
+            cnt = np.array([11], np.uint32)
+            paths = (C.c_uint32 * 4)()
+            stride = int(fn.rsplit("_", 1)[1]) if "stride" in fn else 0
+            hostsim.lib.hs_loss_wave(C.byref(a), ptr(tgt), n_active, ptr(idx), ptr(dt), ptr(coords), ptr(comp), ptr(cnt), ptr(net), ptr(dloss),
+                                     ptr(loss), ptr(rgb), paths, stride)
+            tot = int(cnt[0])
+            in_window, chunked, per_ray, several = paths[0], paths[1], paths[2], paths[3]
+            table_overflows = stride != 0 and int(base[n_active - 1] - base[0]) // stride + 1 > n_rays // 16 + 64    # (a forced stride can ask for more items than the table holds)
+            if kind == "shuffled" or table_overflows:
+                assert in_window == 0 and chunked == 0 and per_ray == (n_active + 63) // 64
+            else:
+                assert per_ray == 0 and in_window > 0
+                if kind == "long":
+                    assert chunked > 0
+                if stride == 4096:
+                    assert several > 0      # more than 64 rays start in windows of that size
+                if stride == 0 and kind in ("short", "split", "gaps"):
+                    assert several == 0 and chunked == 0
         else:
             cnt = np.array([11], np.uint32)
             ns, nm = C.c_uint32(), C.c_uint32()
@@ -95,13 +115,18 @@ def test_fused_handles_empty_and_inactive_batches(orc, hostsim):
         tgt = rng.random((n_rays, 4)).astype(np.float32)
         a = loss_args(n_rays, max(total, 1))
         res = []
-        for fn in ("oracle", "fused"):
+        for fn in ("oracle", "fused", "wave"):
             idx = np.stack([counts, base], axis=1).astype(np.uint32)
             dloss = np.zeros((max(total, 1), 4), np.float32)
             loss = np.full(n_rays, -1, np.float32)
             rgb = np.zeros((n_rays, 3), np.float32)
             if fn == "oracle":
                 tot = orc.volume_rendering_with_loss_and_gradient(a, tgt, n_active, idx, dt, net, dloss, loss_output=loss, rgb_ray_out=rgb)
+            elif fn == "wave":
+                cnt = np.array([0], np.uint32)
+                paths = (C.c_uint32 * 4)()
+                hostsim.lib.hs_loss_wave(C.byref(a), ptr(tgt), n_active, ptr(idx), ptr(dt), None, None, ptr(cnt), ptr(net), ptr(dloss), ptr(loss), ptr(rgb), paths, 0)
+                tot = int(cnt[0])
             else:
                 cnt = np.array([0], np.uint32)
                 ns, nm = C.c_uint32(), C.c_uint32()

@@ -516,7 +516,7 @@ def test_loss_and_gradient(gpu, orc, hin, hout, variant):
 
 
 @pytest.mark.parametrize("loss", ["L1", "Mape", "Smape", "SmoothL1", "LogL1", "RelativeL2"])
-@pytest.mark.parametrize("impl", ["stream", "unfused"])
+@pytest.mark.parametrize("impl", ["waves", "stream", "unfused"])
 def test_every_loss_function(gpu, orc, loss, impl, monkeypatch):
     """loss.cu:27-84: the six losses besides L2, through both compositing implementations, with sRGB targets, a visible background
     and a capacity that clamps the last rays"""
@@ -917,13 +917,14 @@ def test_errors_are_reported_not_thrown_across_the_abi(gpu):
         s.init(1, (4, 4), (1.0, 1.0), (0.5, 0.5), None, None, api.Pcg32(1))
 
 
+@pytest.mark.parametrize("impl", ["waves", "stream"])
 @pytest.mark.parametrize("acts", ["plain", "activated"])
 @pytest.mark.parametrize("kind", ["short", "long", "split", "tiny", "gaps", "biggap", "shuffled"])
-def test_single_launch_compositing_layouts(gpu, orc, kind, acts, monkeypatch):
+def test_single_launch_compositing_layouts(gpu, orc, kind, acts, impl, monkeypatch):
     """every sample layout the streaming compositing distinguishes (back-to-back rays, holes, groups longer than a window,
     shuffled offsets), against the oracle, over many workgroups so that its ordered offsets really go through the chain;
     with the activations compiled out ("plain": both None) and with the run-time switches (Logistic colour, Exponential density)"""
-    monkeypatch.delenv("SRF_COMPOSITE_IMPL", raising=False)
+    monkeypatch.setenv("SRF_COMPOSITE_IMPL", impl)
     rgb_act, den_act = (O.ACT_NONE, O.ACT_NONE) if acts == "plain" else (O.ACT_LOGISTIC, O.ACT_EXPONENTIAL)
     torch = gpu
     from sphericalrf_amd import api
@@ -1032,7 +1033,7 @@ def test_single_launch_and_three_launch_compositing_agree_at_full_size(gpu, orc,
     nrc = torch.full((1,), n_rays, dtype=torch.int32, device="cuda")
     mean_t = torch.ones(1, device="cuda")
     outs = []
-    for reg, impl in (("None", "unfused"), ("None", "stream"), ("Distortion", "stream")):
+    for reg, impl in (("None", "unfused"), ("None", "waves"), ("None", "stream"), ("Distortion", "stream")):
         monkeypatch.setenv("SRF_COMPOSITE_IMPL", impl)
         m = api.RayMarcher(dict(train_with_random_bg_color=False, train_in_linear_color=True, regularization_type=reg))
         idx = idx0.clone()
