@@ -39,7 +39,7 @@ struct ChainScratch {
 	uint32_t* disorder;                 // set when the call's rays are not laid out in increasing order
 	uint32_t* exits;                    // workgroups that have left
 	uint32_t* stride;                   // stride of the sample windows
-	uint32_t* item_first;               // per item: its first ray; one more entry: the number of active rays
+	void* item_desc;                    // per item: its rays and samples (wv::ItemDesc)
 	void* args_copy;                    // the call's fused::Args and this structure, in device memory
 	void* scratch_copy;
 };
@@ -78,11 +78,12 @@ __device__ inline void chain_publish(const ChainScratch& S, uint32_t i, uint32_t
 // entries so that its successors stop at once, raises the error words and returns CHAIN_FAILED.
 struct ChainPeek { unsigned long long vg, vs, vp; uint32_t initial; };
 
-__device__ inline ChainPeek chain_peek(const ChainScratch& S, uint32_t i) {
+// initial: *S.initial, for a caller that has read it already
+__device__ inline ChainPeek chain_peek(const ChainScratch& S, uint32_t i, uint32_t initial) {
 	const uint32_t lane = lane_id();
 	const uint32_t seg = i / WAVE, j = i % WAVE;
 	ChainPeek p;
-	p.initial = *S.initial;
+	p.initial = initial;
 	p.vg = 1ull << 32;
 	if (j != 0 && lane < j) p.vg = status_load(&S.item_status[seg * WAVE + lane]);
 	p.vs = 0ull;
@@ -91,6 +92,8 @@ __device__ inline ChainPeek chain_peek(const ChainScratch& S, uint32_t i) {
 	if (idx >= 0) { p.vs = status_load(&S.seg_status[(size_t)idx * SEG_STRIDE]); p.vp = status_load(&S.seg_prefix[idx]); }
 	return p;
 }
+
+__device__ inline ChainPeek chain_peek(const ChainScratch& S, uint32_t i) { return chain_peek(S, i, *S.initial); }
 
 __device__ inline uint32_t chain_resolve(const ChainScratch& S, uint32_t i, uint32_t total, const ChainPeek& peek) {
 	const uint32_t lane = lane_id();

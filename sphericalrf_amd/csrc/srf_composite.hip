@@ -319,8 +319,9 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 	const uint32_t counter_now = *n_rays_counter;
 	A.mean_density = mean_density_ptr ? *mean_density_ptr : 0.f;
 	A.n_active = counter_now < A.K.n_rays ? counter_now : A.K.n_rays;   // rays past the active count belong to no item: they are left untouched
-	const uint32_t n_items = *S.n_items;
+	const uint32_t n_items = SRF_UNIFORM_U32(*S.n_items);
 	if (blockIdx.x >= n_items) return;
+	const uint32_t initial = SRF_UNIFORM_U32(*S.initial);     // (in a scalar register: looked at in the loop, it is not waited for again there)
 
 #ifdef SRF_KERNEL_TIMING
 	unsigned long long t_acc_[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -445,7 +446,7 @@ __global__ void __launch_bounds__(STREAM_THREADS) SRF_STREAM_OCCUPANCY k_composi
 				chain_publish(S, i_1, total_cur);
 				SRF_T(7);
 				if (fast1) chain_counted<G, false>(lane, n_cur, wave_max_fast(n_cur), w1, sh.rl, pl1, carry);
-				peek = chain_peek(S, i_1);                            // needed in the next first half; the items before this one have published by now unless their workgroups lag
+				peek = chain_peek(S, i_1, initial);                            // needed in the next first half; the items before this one have published by now unless their workgroups lag
 				SRF_T(4);
 			}
 		} else if (plan_wave) {
@@ -589,9 +590,10 @@ __global__ void __launch_bounds__(256) k_fill_rollover_rescale(uint32_t n_elemen
 static int check_chain_error(srf_marcher* m) {
 	if (m->host_error && *m->host_error) {
 		*m->host_error = 0u;
-		m->degraded = true;
+		m->degraded += 1;
 		SRF_FAIL(SRF_ERR_HIP, "compositing: in an earlier call a workgroup gave up waiting for its predecessors' sample counts; that call's compacted "
-		                      "offsets and gradients are invalid (its compacted counter reads 0xffffffff). This marcher now uses the three-launch implementation.");
+		                      "offsets and gradients are invalid (its compacted counter reads 0xffffffff). This marcher now uses %s.",
+		         m->degraded == 1 && !m->force_waves ? "the wave-per-item kernel" : "the three-launch implementation");
 	}
 	return SRF_OK;
 }
@@ -786,7 +788,7 @@ int srf_marcher_create(const srf_marcher_config* cfg, srf_marcher_t** out) {
 	// call on this marcher; the tests use it to compare the two implementations
 	const char* impl_env = getenv("SRF_COMPOSITE_IMPL");
 	m->force_unfused = impl_env && strcmp(impl_env, "unfused") == 0;
-	m->force_stream = !(impl_env && strcmp(impl_env, "waves") == 0);      // (until the wave-per-item kernel is the faster one)
+	m->force_waves = impl_env && strcmp(impl_env, "waves") == 0;
 	// A word of host memory that the device can write: the streaming kernel raises it when its ordered-offset chain gives up, and
 	// the next call reads it without waiting for the device.  Without a device (configuration-only use) there is none.
 	int n_dev = 0;
@@ -849,17 +851,21 @@ int srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const 
 	rc = check_chain_error(m);
 	if (rc != SRF_OK) return rc;
 	// The distortion regulariser's side buffer is only filled by the three-launch implementation, which also serves a marcher
-	// whose chain has failed before, and one created under SRF_COMPOSITE_IMPL=unfused.
-	if (m->cfg.regularization_type != SRF_REG_DISTORTION && !m->force_unfused && !m->force_stream && !m->degraded) {
+	// created under SRF_COMPOSITE_IMPL=unfused and one whose chain has failed in both single-launch kernels.
+	// The streaming kernel by default.  The wave-per-item kernel where asked for (SRF_COMPOSITE_IMPL=waves) and after the streaming
+	// kernel's chain has given up once (its items wait for workgroups that must all be running; the wave-per-item kernel's never do).
+	const bool fusable = m->cfg.regularization_type != SRF_REG_DISTORTION && !m->force_unfused;
+	const int level = m->degraded + (m->force_waves ? 1 : 0);
+	if (fusable && level == 1) {
 		const void* before = m->wave_ws.ptr;
 		rc = m->wave_ws.reserve(waves_scratch_bytes(a->n_rays));
 		if (rc != SRF_OK) return rc;
 		if (m->wave_ws.ptr != before) SRF_HIP(hipMemsetAsync(m->wave_ws.ptr, 0, 512, st));      // a new buffer: the words that are zero between calls
 		m->chain_error_dev = waves_error_word(m->wave_ws.ptr);
-		return launch_waves(a, K, m->wave_ws.ptr, m->host_error_dev, m->lookback_spin_limit, rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
+		return launch_waves(a, K, m->wave_ws.ptr, m->host_error_dev, m->force_waves ? m->lookback_spin_limit : (1u << 22), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
 		                    compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, st);
 	}
-	if (m->cfg.regularization_type != SRF_REG_DISTORTION && !m->force_unfused && !m->degraded) {
+	if (fusable && level == 0) {
 		rc = m->ws.reserve(chain_layout(a->n_rays).bytes);
 		if (rc != SRF_OK) return rc;
 		m->chain_error_dev = chain_scratch_at(m->ws.ptr, a->n_rays, nullptr, 0).error;
@@ -916,7 +922,7 @@ int srf_marcher_volume_rendering_with_loss_and_gradient_noalloc(srf_marcher_t* m
 	SRF_REQUIRE(m->cfg.regularization_type != SRF_REG_DISTORTION, "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: the distortion regulariser needs buffers that this entry point may not allocate");
 	rc = check_chain_error(m);
 	if (rc != SRF_OK) return rc;
-	SRF_REQUIRE(!m->force_unfused && !m->degraded, "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: this marcher uses the three-launch implementation, which allocates");
+	SRF_REQUIRE(!m->force_unfused && !m->force_waves && !m->degraded, "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: this marcher no longer uses the streaming kernel; the other implementations allocate");
 	void* scratch = nullptr;
 	rc = noalloc_scratch(&scratch);
 	if (rc != SRF_OK) return rc;
@@ -931,14 +937,14 @@ int srf_marcher_sync_check(srf_marcher_t* m, void* stream) {
 	if (m->chain_error_dev) {
 		uint32_t flag = 0;
 		SRF_HIP(hipMemcpy(&flag, m->chain_error_dev, 4, hipMemcpyDeviceToHost));
-		if (flag) {      // reported once: the word is cleared, and no later call of this marcher writes it (it has fallen back)
+		if (flag) {      // reported once: the word is cleared, and the marcher's next call uses the next implementation, with an error word of its own
 			const uint32_t zero = 0;
 			SRF_HIP(hipMemcpy(m->chain_error_dev, &zero, 4, hipMemcpyHostToDevice));
 			m->chain_error_dev = nullptr;
 		}
 		if (flag && m->host_error) *m->host_error = 1u;
 		if (flag && !m->host_error) {
-			m->degraded = true;
+			m->degraded += 1;
 			SRF_FAIL(SRF_ERR_HIP, "compositing: a workgroup gave up waiting for its predecessors' sample counts; compacted offsets of the last call are invalid");
 		}
 	}

@@ -81,8 +81,9 @@ struct srf_marcher {
 	unsigned long long* frame_word_dev = nullptr;   // device address of the second of them (8 bytes in), which the compaction kernel writes itself
 	uint32_t frame_stamp = 0;                // number of the last compaction srf_render_frame waited for
 	bool force_unfused = false;             // SRF_COMPOSITE_IMPL=unfused at creation
-	bool force_stream = false;              // SRF_COMPOSITE_IMPL=stream at creation
-	bool degraded = false;                  // the chain has failed once: every later call uses the three-launch implementation
+	bool force_waves = false;               // SRF_COMPOSITE_IMPL=waves at creation
+	int degraded = 0;                       // how often a chain of ordered offsets has given up: after the first time the wave-per-item kernel (whose items never wait
+	                                        // for a workgroup that is not running) takes the calls, after the second the three-launch implementation
 	volatile uint32_t* host_error = nullptr; // host word the streaming kernel raises when its chain gives up (pinned, device-writable)
 	uint32_t* host_error_dev = nullptr;      // the same word as the device addresses it
 	uint32_t* chain_error_dev = nullptr;     // device word of the last streaming launch (NULL before the first)

@@ -9,6 +9,7 @@ static uint64_t g_radius_hist[8][4] = {};   // [cascade][radius 0, 1-block, 2-3,
 #define SRF_COUNT_RADIUS(n, level) (++g_radius_hist[(level) & 7][(n) == 0 ? 0 : ((n) >> (level)) <= 1 ? 1 : ((n) >> (level)) <= 3 ? 2 : 3])
 #include <cstring>
 #include <vector>
+#include <array>
 #include <cstdlib>
 #include <algorithm>
 #include "../../sphericalrf_amd/csrc/srf_bodies.h"
@@ -206,9 +207,10 @@ static void run_wave(const orc_loss_args* a, const float* rays_rgba, uint32_t n_
 	// preparing pass
 	Windows W = windows_of(A.n_active, ray_coord_indices, cap);
 	if (force_stride) { W.stride = force_stride; W.n_items = A.n_active ? (uint32_t)((ray_coord_indices[2 * (size_t)(A.n_active - 1) + 1] - W.base0) / W.stride) + 1 : 0; }
-	std::vector<uint32_t> item_first((size_t)cap + 1, 0xdeadbeefu);
+	std::vector<ItemDesc> desc((size_t)cap);
+	std::memset(desc.data(), 0xdb, desc.size() * sizeof(ItemDesc));
 	bool irregular = false;
-	for (uint32_t i = 0; i < A.n_active; ++i) if (!prepare_ray(i, A.n_active, ray_coord_indices, W, cap, item_first.data())) irregular = true;
+	for (uint32_t i = 0; i < A.n_active; ++i) if (!prepare_ray(i, A.n_active, ray_coord_indices, W, cap, desc.data())) irregular = true;
 	if (!irregular && W.n_items > cap) irregular = true;      // (a forced stride may ask for more items than the table holds)
 	const uint32_t n_items = irregular ? (A.n_active + GROUP - 1) / GROUP : W.n_items;
 	Lds* wp = new Lds();
@@ -274,10 +276,32 @@ static void run_wave(const orc_loss_args* a, const float* rays_rgba, uint32_t n_
 	for (uint32_t item = 0; item < n_items; ++item) {
 		uint32_t r0, n_r;
 		if (irregular) { r0 = item * GROUP; n_r = A.n_active - r0 < GROUP ? A.n_active - r0 : GROUP; }
-		else { r0 = item_first[item]; n_r = item_first[item + 1] - r0; }
+		else { r0 = desc[item].r0; n_r = desc[item].r_end - r0; }
 		if (!irregular) {
 			const uint32_t n_batches = (n_r + LANES - 1) / LANES;
-			if (n_batches <= 1) {
+			if (n_batches <= 1 && desc[item].s_end - desc[item].s0 <= WIN) {
+				// the common item: in one piece, with the gradients staged in the window before the item's offset is looked at
+				++counts[0];
+				load_batch(r0, n_r);
+				if (B.s0 != desc[item].s0 && n_r) std::abort();
+				if (B.range != desc[item].s_end - desc[item].s0) std::abort();
+				std::vector<RowData<HI>> in(LANES);
+				std::vector<std::array<float, ROWS>> alpha(LANES);
+				RayLds2& rl = w.staged();
+				if (B.range) for (uint32_t l = 0; l < LANES; ++l) fit_rows_load<HI>(l, A, B.s0, B.range, in[l]);
+				for (uint32_t l = 0; l < LANES; ++l) { if (plain) fit_rows_alpha<HI, true>(l, A, w.S, w.owner, B.range, in[l], alpha[l].data()); else fit_rows_alpha<HI, false>(l, A, w.S, w.owner, B.range, in[l], alpha[l].data()); }
+				for (uint32_t l = 0; l < LANES; ++l) ray_reset(B.rs[l]);
+				chain_all(0);
+				float loss[LANES];
+				for (uint32_t l = 0; l < B.nb; ++l) loss[l] = fit_finish_lane(l, B.rb + l, B.n[l], A, rl, B.rs[l], B.tgt[l]);
+				for (uint32_t l = 0; l < LANES; ++l) { if (plain) fit_rows_grads<HI, true>(l, A, w.S, w.owner, rl, B.range, in[l], alpha[l].data()); else fit_rows_grads<HI, false>(l, A, w.S, w.owner, rl, B.range, in[l], alpha[l].data()); }
+				uint32_t run = prefix;        // (the device publishes the total before the gradients and chains it to the earlier items' after them)
+				for (uint32_t l = 0; l < LANES; ++l) {
+					if (l < B.nb) { fit_commit_lane(l, B.rb + l, B.rs[l].cnt, B.rbase[l], run, prefix, loss[l], A, rl); run += B.rs[l].cnt; } else fit_commit_none(l, rl);
+				}
+				for (uint32_t l = 0; l < LANES; ++l) fit_rows_store<HO>(l, A, w.S, w.owner, rl, B.s0, B.range, prefix);
+				prefix = run;
+			} else if (n_batches <= 1) {
 				load_batch(r0, n_r);
 				forward();
 				const uint32_t total = batch_total();
