@@ -44,6 +44,10 @@ enum { SRF_DTYPE_F16 = 0, SRF_DTYPE_F32 = 1 };
 
 typedef struct srf_sampler srf_sampler_t;   /* OccupancySampler, internal/sampler/occupancy_sampler.h:13-135 */
 typedef struct srf_marcher srf_marcher_t;   /* RayMarcher,       internal/render/ray_marcher.h:13-81 */
+/* Threads and streams: a handle owns workspaces that its calls reuse without locking, as the reference's objects own their
+ * GPUMemory members.  Use one handle from one thread at a time, and keep its calls on one stream (or order the streams yourself
+ * with events): two calls on one handle that overlap on the device share those workspaces and race.  Different handles are
+ * independent, except for srf_marcher_volume_rendering_with_loss_and_gradient_noalloc (see there). */
 
 /* tcnn::pcg32 state; callers keep it on the host exactly as Testbed::m_rng does (internal/testbed.h:92-93) */
 typedef struct srf_pcg32 { uint64_t state, inc; } srf_pcg32;
@@ -155,6 +159,9 @@ int  srf_ray_sphere_bounds(uint32_t n_rays, const float* rays, const float cente
 
 /* Testbed::load_snapshot, internal/testbed.cu:167: overwrite density_grid (n_total_elements floats, device) */
 int  srf_sampler_set_density_grid(srf_sampler_t* s, const float* density_grid, void* stream);
+/* The two sampler lines of Testbed::load_snapshot, internal/testbed.cu:166-167: density_grid is assigned from the snapshot's values
+ * in host memory (n_values must be n_total_elements) and the bitfield is rebuilt.  Returns when the copy has finished. */
+int  srf_sampler_load_density_grid(srf_sampler_t* s, const float* density_grid_host, uint32_t n_values, void* stream);
 
 /* No counterpart in the reference: the order in which srf_sampler_sample_positions_from_grid hands the uniform points over.
  * 0 (default): the reference's, point i in entry i.  1, cell order: with a power-of-two cell count n_cells (at least 2048) the
@@ -247,9 +254,14 @@ int  srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It runs the single-launch implementation with its
  * scratch (the per-item status words, item lists and per-ray side array of the ordered-offset chain) in an array that is part of
  * the library's device image, about 1.3 MB on every GPU the library runs on, and calls no hipMalloc / hipFree.
- * Limits: n_rays <= SRF_NOALLOC_MAX_RAYS; no distortion regulariser; refused on a marcher that has fallen back to the
- * three-launch implementation.  All calls on one GPU share the array: calls that overlap on one GPU (different streams or
- * threads) race.  Arguments, results and error reporting are those of srf_marcher_volume_rendering_with_loss_and_gradient.
+ * Limits: n_rays <= SRF_NOALLOC_MAX_RAYS; no distortion regulariser; refused on a marcher that has left the streaming kernel
+ * (after a failed chain, or created under SRF_COMPOSITE_IMPL).  All calls on one GPU, of whatever marcher, share the array and
+ * the chain's error word in it: at most one such call may be in flight per GPU, and calls that overlap on one GPU (different
+ * streams or threads) race.  Because the next call's preparation clears the shared error word, a marcher without a host-visible
+ * error word of its own must call srf_marcher_sync_check before another marcher uses this entry point on the same GPU.
+ * The first call on a device, and the first for each combination of data types and activations, does host-side look-ups (the
+ * array's address, the kernel's occupancy): make those calls before a graph capture begins, not inside one.
+ * Arguments, results and error reporting are those of srf_marcher_volume_rendering_with_loss_and_gradient.
  */
 #define SRF_NOALLOC_MAX_RAYS 262144u
 int  srf_marcher_volume_rendering_with_loss_and_gradient_noalloc(srf_marcher_t* m, const srf_loss_args* args,
@@ -272,7 +284,9 @@ typedef struct srf_render_args {
  * The streaming kernel's workgroups wait, with a bound, for the sample counts of the groups before theirs.  If a wait runs
  * out, that call's compacted counter reads 0xffffffff, every ray of the affected groups gets a zero count and no gradients, and
  * the failure is returned by this function or by the next srf_marcher_volume_rendering_with_loss_and_gradient on the marcher,
- * whichever comes first; from then on the marcher uses the three-launch implementation, which has no such waits. */
+ * whichever comes first; from then on the marcher uses the wave-per-item kernel, whose items are handed out by a counter and so
+ * never wait for a workgroup that is not running (and, should that kernel's waits run out as well, the three-launch
+ * implementation, which has none). */
 int  srf_marcher_sync_check(srf_marcher_t* m, void* stream);
 
 /* RayMarcher::volume_rendering, ray_marcher.cu:376-415 (kernel :204-282) */
@@ -315,6 +329,12 @@ int  srf_field_eval(const srf_sampler_t* s, const srf_field* field, uint32_t n_c
  * (any other value is reported as SRF_ERR_INVALID). */
 typedef int (*srf_inference_fn)(void* user, uint32_t n_elements, const float* coords, void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream);
 
+/* What the caller's network does in Normals mode between inference and srf_marcher_volume_rendering
+ * (m_network->input_gradient(stream, 3, coords, coords), internal/testbed.cu:558-560): the first three floats of each of the
+ * n_elements coordinate records are overwritten with the density's gradient with respect to them, enqueued on `stream`.
+ * Returns like srf_inference_fn. */
+typedef int (*srf_input_gradient_fn)(void* user, uint32_t n_elements, float* coords, void* stream);
+
 typedef struct srf_frame_args {
 	int32_t  resolution[2];
 	float    focal_length[2], principal_point[2];
@@ -324,19 +344,25 @@ typedef struct srf_frame_args {
 	float    depth_scale;                /* 1 / scene_scale (testbed.cu:577) */
 	int32_t  network_output_dtype;
 	uint32_t padded_output_width;
+	srf_input_gradient_fn input_gradient; /* called after inference when render_mode is SRF_RENDER_NORMALS (which is refused with */
+	void*    input_gradient_user;         /* SRF_ERR_UNSUPPORTED when this is NULL); ignored in every other mode */
 } srf_frame_args;
 
 /* Testbed::render_frame up to and including shade_kernel, internal/testbed.cu:479-611: rays from the camera, then rounds of
  * compact_rays / generate_coords_from_rays / inference / volume_rendering with n_steps = clamp(n_pixels / n_alive, 1, 8) until no ray
  * is alive, then shade into frame_buffer (4 floats a pixel, cleared first).  The marcher owns the ray, coordinate and network-output
- * buffers.  Like the reference it waits for the stream once a round to read the number of rays left.  *n_iterations (may be NULL)
- * receives the number of rounds. */
+ * buffers.  Like the reference the host learns the number of rays left once a round: the compaction's last workgroup stores it into
+ * mapped host memory and the calling thread polls that word (a busy wait on one host core, with hipStreamQuery every 4096 polls and a
+ * copy plus hipStreamSynchronize should the word not arrive).  *n_iterations (may be NULL) receives the number of rounds. */
 int  srf_render_frame(srf_sampler_t* s, srf_marcher_t* m, const srf_frame_args* args, srf_inference_fn inference, void* user,
                       float* frame_buffer, uint32_t* n_iterations, void* stream);
 
 /* an srf_inference_fn that evaluates the stand-in field (srf_field_eval); user points at an srf_field_inference_ctx */
 typedef struct srf_field_inference_ctx { const srf_sampler_t* sampler; const srf_field* field; } srf_field_inference_ctx;
 int  srf_field_inference(void* user, uint32_t n_elements, const float* coords, void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream);
+/* an srf_input_gradient_fn for the stand-in field (user as above): the position of each record becomes the first three values,
+ * minus one half, of the table row that the field with seed ^ 0x9e3779b9 selects for it */
+int  srf_field_input_gradient(void* user, uint32_t n_elements, float* coords, void* stream);
 
 /* CudaRenderBuffer::accumulate, internal/utils/render_buffer.cu:46-85, :211-227: running mean of the frames of one view.  spp is the
  * number of frames already accumulated (0: the buffer is cleared first); the caller counts. */

@@ -163,6 +163,7 @@ class Oracle:
         L.orc_grid_mean.argtypes = [vp, u32]
         L.orc_update_grid_bitfield.restype = f32
         L.orc_render_frame.restype = u32
+        L.orc_render_frame_mode.restype = u32
 
     # ---- primitives -------------------------------------------------------------
     def max_threads(self):
@@ -429,14 +430,14 @@ class Oracle:
                              int(curve), _ptr(out))
         return out
 
-    def render_frame(self, p, field, bitfield, res, focal, pp, cam, spp=0, transmittance_threshold=1e-4, train_in_linear_colors=True):
+    def render_frame(self, p, field, bitfield, res, focal, pp, cam, spp=0, transmittance_threshold=1e-4, train_in_linear_colors=True, render_mode=RENDER_SHADE):
         n = res[0] * res[1]
         frame = np.zeros((res[1], res[0], 4), np.float32)
         nsamp = np.zeros(n, np.uint32)
         cam = np.ascontiguousarray(cam, dtype=np.float32).ravel()
-        iters = self.lib.orc_render_frame(C.byref(p), C.byref(field), _ptr(bitfield, np.uint8, allow_none=not p.use_grid),
-                                          (i32 * 2)(*res), (f32 * 2)(*focal), (f32 * 2)(*pp), _ptr(cam, np.float32, 12), u32(spp),
-                                          f32(transmittance_threshold), int(train_in_linear_colors), _ptr(frame), _ptr(nsamp))
+        iters = self.lib.orc_render_frame_mode(C.byref(p), C.byref(field), _ptr(bitfield, np.uint8, allow_none=not p.use_grid),
+                                               (i32 * 2)(*res), (f32 * 2)(*focal), (f32 * 2)(*pp), _ptr(cam, np.float32, 12), u32(spp),
+                                               f32(transmittance_threshold), int(train_in_linear_colors), int(render_mode), _ptr(frame), _ptr(nsamp))
         return frame, nsamp.reshape(res[1], res[0]), int(iters)
 
 

@@ -521,6 +521,10 @@ inline float network_to_rgb(float v, int act) {
 	}
 	return 0.0f;
 }
+// fmaxf(0.0f, x) as CUDA evaluates it (ray_marcher.cu:187-189): its max orders -0 below +0, so either zero gives +0; NaN gives 0.
+// The C library's fmaxf leaves that sign open.
+inline float max_zero(float x) { return x > 0.0f ? x : 0.0f; }
+
 inline float network_to_rgb_derivative(float v, int act) {
 	switch (act) {
 	case ORC_ACT_NONE: return 1.0f;
@@ -1283,9 +1287,9 @@ void orc_volume_rendering_with_loss_and_gradient(const orc_loss_args* A,
 			T *= (1.f - alpha);
 			const V3 dloss_by_drgb = weight * g;
 			float out[4];
-			out[0] = loss_scale * (dloss_by_drgb.x * network_to_rgb_derivative(raw[0], a.rgb_activation) + fmaxf(0.0f, output_l2_reg * raw[0]));
-			out[1] = loss_scale * (dloss_by_drgb.y * network_to_rgb_derivative(raw[1], a.rgb_activation) + fmaxf(0.0f, output_l2_reg * raw[1]));
-			out[2] = loss_scale * (dloss_by_drgb.z * network_to_rgb_derivative(raw[2], a.rgb_activation) + fmaxf(0.0f, output_l2_reg * raw[2]));
+			out[0] = loss_scale * (dloss_by_drgb.x * network_to_rgb_derivative(raw[0], a.rgb_activation) + max_zero(output_l2_reg * raw[0]));
+			out[1] = loss_scale * (dloss_by_drgb.y * network_to_rgb_derivative(raw[1], a.rgb_activation) + max_zero(output_l2_reg * raw[1]));
+			out[2] = loss_scale * (dloss_by_drgb.z * network_to_rgb_derivative(raw[2], a.rgb_activation) + max_zero(output_l2_reg * raw[2]));
 			const V3 suffix = f.rgb_ray - rgb_ray2;
 			const float density_derivative = network_to_density_derivative(raw[3], a.density_activation);
 			const float dloss_by_dmlp = density_derivative * (dt * dot3(g, T * rgb - suffix));
@@ -1507,6 +1511,23 @@ void orc_field_eval(const orc_params* Pp, const orc_field* f, const float wpos[3
 uint32_t orc_render_frame(const orc_params* Pp, const orc_field* f, const uint8_t* bitfield,
                           const int32_t res[2], const float focal[2], const float pp[2], const float cam[12],
                           uint32_t spp, float transmittance_threshold, int train_in_linear_colors, float* frame, uint32_t* n_samples_per_pixel) {
+	return orc_render_frame_mode(Pp, f, bitfield, res, focal, pp, cam, spp, transmittance_threshold, train_in_linear_colors, ORC_RENDER_SHADE, frame, n_samples_per_pixel);
+}
+
+// Stand-in for NGPNetwork::input_gradient (the density's gradient with respect to the position): a second row of the table,
+// centred on zero, replaces the sample's position.  Not in the reference.
+void orc_field_input_gradient(const orc_params* Pp, const orc_field* f, float* coord) {
+	const orc_field g{f->table, f->table_size, f->seed ^ 0x9e3779b9u};
+	float row[4];
+	orc_field_eval(Pp, &g, coord, row);
+	coord[0] = row[0] - 0.5f; coord[1] = row[1] - 0.5f; coord[2] = row[2] - 0.5f;
+}
+
+// the same loop in any render mode; in Normals mode the coordinates of a round are overwritten with the density's input gradient
+// between inference and volume_rendering (internal/testbed.cu:558-560)
+uint32_t orc_render_frame_mode(const orc_params* Pp, const orc_field* f, const uint8_t* bitfield,
+                               const int32_t res[2], const float focal[2], const float pp[2], const float cam[12],
+                               uint32_t spp, float transmittance_threshold, int train_in_linear_colors, int render_mode, float* frame, uint32_t* n_samples_per_pixel) {
 	const orc_params& P = *Pp;
 	const uint32_t n_pixels = (uint32_t)res[0] * (uint32_t)res[1];
 	std::vector<orc_payload> pay[2] = {std::vector<orc_payload>(n_pixels), std::vector<orc_payload>(n_pixels)};
@@ -1542,6 +1563,7 @@ uint32_t orc_render_frame(const orc_params* Pp, const orc_field* f, const uint8_
 			for (uint32_t j = 0; j < pcur[i].n_steps; ++j) {
 				size_t s = (size_t)i * n_steps + j;
 				orc_field_eval(Pp, f, coords.data() + 7 * s, rgbsigma.data() + 4 * s);
+				if (render_mode == ORC_RENDER_NORMALS) orc_field_input_gradient(Pp, f, coords.data() + 7 * s);
 			}
 		}
 		std::vector<uint8_t> was_alive(n_alive);
@@ -1549,7 +1571,7 @@ uint32_t orc_render_frame(const orc_params* Pp, const orc_field* f, const uint8_
 		orc_render_args ra;
 		memset(&ra, 0, sizeof(ra));
 		ra.n_rays = n_alive; ra.n_steps = n_steps; ra.n_steps_offset = i_steps_offset; ra.padded_output_width = 4;
-		ra.density_activation = ORC_ACT_NONE; ra.rgb_activation = ORC_ACT_NONE; ra.render_mode = ORC_RENDER_SHADE;
+		ra.density_activation = ORC_ACT_NONE; ra.rgb_activation = ORC_ACT_NONE; ra.render_mode = render_mode;
 		memcpy(ra.camera, cam, sizeof(ra.camera));
 		ra.depth_scale = 1.f; ra.transmittance_threshold = transmittance_threshold; ra.network_output_dtype = ORC_DTYPE_F32;
 		orc_volume_rendering(Pp, &ra, pcur.data(), ccur.data(), coords.data(), rgbsigma.data());
@@ -1569,7 +1591,7 @@ uint32_t orc_render_frame(const orc_params* Pp, const orc_field* f, const uint8_
 		}
 		i_steps_offset += n_steps;
 	}
-	orc_shade(n_hit, hit_col.data(), hit_pay.data(), frame, ORC_RENDER_SHADE, train_in_linear_colors);
+	orc_shade(n_hit, hit_col.data(), hit_pay.data(), frame, render_mode, train_in_linear_colors);
 	return iters;
 }
 

@@ -210,6 +210,13 @@ uint32_t orc_render_frame(const orc_params* p, const orc_field* f, const uint8_t
                           const int32_t res[2], const float focal[2], const float pp[2], const float cam[12],
                           uint32_t spp, float transmittance_threshold, int train_in_linear_colors,
                           float* frame, uint32_t* n_samples_per_pixel /* may be NULL */);
+/* stand-in for the network's input gradient: overwrites the position of one coordinate record (not in the reference) */
+void  orc_field_input_gradient(const orc_params* p, const orc_field* f, float* coord);
+/* the same loop in a given render mode (internal/testbed.cu:558-560: Normals mode replaces the coordinates by the input gradient) */
+uint32_t orc_render_frame_mode(const orc_params* p, const orc_field* f, const uint8_t* bitfield,
+                               const int32_t res[2], const float focal[2], const float pp[2], const float cam[12],
+                               uint32_t spp, float transmittance_threshold, int train_in_linear_colors, int render_mode,
+                               float* frame, uint32_t* n_samples_per_pixel /* may be NULL */);
 
 #ifdef __cplusplus
 }

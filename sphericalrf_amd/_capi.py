@@ -90,6 +90,7 @@ class FrameArgs(C.Structure):
         ("resolution", i32 * 2), ("focal_length", f32 * 2), ("principal_point", f32 * 2), ("camera_matrix", f32 * 12), ("spp", u32),
         ("render_mode", i32), ("density_activation", i32), ("rgb_activation", i32), ("depth_scale", f32),
         ("network_output_dtype", i32), ("padded_output_width", u32),
+        ("input_gradient", vp), ("input_gradient_user", vp),
     ]
 
 
@@ -99,19 +100,21 @@ class FieldInferenceCtx(C.Structure):
 
 # srf_inference_fn: (user, n_elements, coords, rgbsigma, dtype, padded_output_width, stream) -> int
 INFERENCE_FN = C.CFUNCTYPE(C.c_int, vp, u32, vp, vp, i32, u32, vp)
+# srf_input_gradient_fn: (user, n_elements, coords, stream) -> int
+INPUT_GRADIENT_FN = C.CFUNCTYPE(C.c_int, vp, u32, vp, vp)
 
 
 # every symbol include/srf_hip.h declares
 SYMBOLS = [
     "srf_last_error", "srf_device_count",
     "srf_sampler_config_default", "srf_sampler_create", "srf_sampler_destroy", "srf_sampler_get_info", "srf_sampler_set_runtime",
-    "srf_sampler_init", "srf_sampler_set_density_grid", "srf_sampler_sample_positions_from_grid", "srf_sampler_update_grid",
+    "srf_sampler_init", "srf_sampler_set_density_grid", "srf_sampler_load_density_grid", "srf_sampler_sample_positions_from_grid", "srf_sampler_update_grid",
     "srf_sampler_update_grid_bitfield", "srf_sampler_sample_coords_from_dataset", "srf_sampler_generate_rays_from_camera_matrix",
     "srf_sampler_generate_coords_from_rays", "srf_sampler_set_ray_sphere_bound", "srf_ray_sphere_bounds", "srf_sampler_set_grid_sample_order",
     "srf_marcher_config_default", "srf_marcher_create", "srf_marcher_destroy", "srf_marcher_get_config", "srf_marcher_set_config",
     "srf_marcher_volume_rendering_with_loss_and_gradient", "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc", "srf_marcher_sync_check", "srf_marcher_volume_rendering",
     "srf_compact_rays", "srf_shade", "srf_fill_rollover", "srf_fill_rollover_and_rescale",
-    "srf_render_frame", "srf_field_inference", "srf_frame_accumulate", "srf_frame_tonemap",
+    "srf_render_frame", "srf_field_inference", "srf_field_input_gradient", "srf_frame_accumulate", "srf_frame_tonemap",
     "srf_render_frame_fused", "srf_field_eval", "srf_debug_eval_elem", "srf_marcher_debug_set_lookback_spin_limit",
 ]
 
@@ -148,6 +151,7 @@ def load():
     L.srf_sampler_set_runtime.argtypes = [vp, i32, i32, f32, f32]
     L.srf_sampler_init.argtypes = [vp, u32, P(i32 * 2), P(f32 * 2), P(f32 * 2), vp, P(Pcg32), vp]
     L.srf_sampler_set_density_grid.argtypes = [vp, vp, vp]
+    L.srf_sampler_load_density_grid.argtypes = [vp, vp, u32, vp]
     L.srf_sampler_set_ray_sphere_bound.argtypes = [vp, P(f32 * 3), f32]
     L.srf_sampler_set_grid_sample_order.argtypes = [vp, i32]
     L.srf_ray_sphere_bounds.argtypes = [u32, vp, P(f32 * 3), f32, vp, vp, vp]
@@ -177,6 +181,7 @@ def load():
     L.srf_field_eval.argtypes = [vp, P(Field), u32, vp, vp, i32, u32, vp]
     L.srf_render_frame.argtypes = [vp, vp, P(FrameArgs), vp, vp, vp, P(u32), vp]
     L.srf_field_inference.argtypes = [vp, u32, vp, vp, i32, u32, vp]
+    L.srf_field_input_gradient.argtypes = [vp, u32, vp, vp]
     L.srf_frame_accumulate.argtypes = [P(i32 * 2), vp, vp, u32, i32, vp]
     L.srf_frame_tonemap.argtypes = [P(i32 * 2), f32, P(f32 * 4), vp, i32, i32, i32, vp, vp]
     L.srf_debug_eval_elem.argtypes = [i32, u32, vp, vp, vp, vp]

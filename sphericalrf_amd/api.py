@@ -12,7 +12,8 @@ import torch
 
 from . import _capi as K
 from ._capi import (ACT_EXPONENTIAL, ACT_LOGISTIC, ACT_NONE, ACT_RELU, COLOR_LINEAR, COLOR_SRGB, DTYPE_F16, DTYPE_F32,  # noqa: F401
-                    LOSS_L2, LOSS_SMOOTHL1, RENDER_SHADE, SrfError)
+                    ERR_HIP, ERR_INVALID, ERR_UNSUPPORTED, LOSS_L2, LOSS_SMOOTHL1, RENDER_AO, RENDER_COST, RENDER_DEPTH, RENDER_DISTANCE,
+                    RENDER_NORMALS, RENDER_SHADE, SrfError)
 
 _WARP = {"ngp": K.WARP_NGP, "mipnerf360": K.WARP_MIPNERF360, "donerf": K.WARP_DONERF, "sigmoid": K.WARP_SIGMOID,
          "erp": K.WARP_ERP, "sinusoidalprojection": K.WARP_SINUSOIDAL}
@@ -338,10 +339,12 @@ class OccupancySampler:
 
     def render_frame(self, marcher, inference, resolution, focal_length, principal_point, camera_matrix, frame_buffer, spp=0,
                      render_mode=K.RENDER_SHADE, density_activation=K.ACT_EXPONENTIAL, rgb_activation=K.ACT_LOGISTIC, depth_scale=1.0,
-                     network_output_dtype=K.DTYPE_F16, padded_output_width=4):
+                     network_output_dtype=K.DTYPE_F16, padded_output_width=4, input_gradient=None):
         """Testbed::render_frame up to shade (internal/testbed.cu:479-611).  `inference` is a Field (the stand-in network) or a callable
         (n_elements, coords_ptr, rgbsigma_ptr, dtype, padded_output_width, stream_ptr) -> int that enqueues the network on the stream.
-        Returns the number of rounds."""
+        Normals mode needs `input_gradient` (testbed.cu:558-560): True with a Field (the stand-in's gradient), else a callable
+        (n_elements, coords_ptr, stream_ptr) -> int that overwrites each record's position with the density's gradient.
+        An exception raised by a callable ends the frame and is raised again here.  Returns the number of rounds."""
         a = K.FrameArgs()
         a.resolution, a.focal_length, a.principal_point = (K.i32 * 2)(*resolution), (K.f32 * 2)(*focal_length), (K.f32 * 2)(*principal_point)
         a.camera_matrix = (K.f32 * 12)(*[float(v) for v in camera_matrix])
@@ -349,15 +352,40 @@ class OccupancySampler:
         a.depth_scale, a.network_output_dtype, a.padded_output_width = float(depth_scale), int(network_output_dtype), int(padded_output_width)
         iters = K.u32(0)
         n = resolution[0] * resolution[1]
+        raised = []
+
+        def guarded(fn, *args):
+            # ctypes prints and drops an exception that leaves a callback, and the frame would go on with stale buffers
+            try:
+                return int(fn(*args) or 0)
+            except BaseException as e:      # noqa: B902 - handed back to the caller below
+                raised.append(e)
+                return K.ERR_INVALID
+
+        keep = []
         if isinstance(inference, Field):
             f = inference.as_c()
             ctx = K.FieldInferenceCtx(self._h, C.pointer(f))
-            fn, user, keep = C.cast(self._L.srf_field_inference, C.c_void_p), C.cast(C.pointer(ctx), C.c_void_p), (f, ctx)
+            fn, user = C.cast(self._L.srf_field_inference, C.c_void_p), C.cast(C.pointer(ctx), C.c_void_p)
+            keep += [f, ctx]
+            if input_gradient is True:
+                a.input_gradient, a.input_gradient_user = C.cast(self._L.srf_field_input_gradient, C.c_void_p), user
+                input_gradient = None
         else:
-            cb = K.INFERENCE_FN(lambda user, n_el, coords, out, dtype, width, stream: int(inference(n_el, coords, out, dtype, width, stream) or 0))
-            fn, user, keep = C.cast(cb, C.c_void_p), None, (cb,)
-        K.check(self._L.srf_render_frame(self._h, marcher._h, C.byref(a), fn, user, _dev(frame_buffer, torch.float32, 4 * n, "frame_buffer"), C.byref(iters), _stream()))
+            cb = K.INFERENCE_FN(lambda user, n_el, coords, out, dtype, width, stream: guarded(inference, n_el, coords, out, dtype, width, stream))
+            fn, user = C.cast(cb, C.c_void_p), None
+            keep.append(cb)
+        if input_gradient is True:
+            raise ValueError("input_gradient=True needs a Field as the inference")
+        if input_gradient is not None:
+            gcb = K.INPUT_GRADIENT_FN(lambda user, n_el, coords, stream: guarded(input_gradient, n_el, coords, stream))
+            a.input_gradient = C.cast(gcb, C.c_void_p)
+            keep.append(gcb)
+        rc = self._L.srf_render_frame(self._h, marcher._h, C.byref(a), fn, user, _dev(frame_buffer, torch.float32, 4 * n, "frame_buffer"), C.byref(iters), _stream())
         del keep
+        if raised:
+            raise raised[0]
+        K.check(rc)
         return int(iters.value)
 
 

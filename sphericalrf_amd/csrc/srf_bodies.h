@@ -377,7 +377,7 @@ SRF_HD void count_begin(CountLane& L, uint32_t i, const Params& P, const CountAr
 	L.o = mk3(0.f, 0.f, 0.f); L.d = L.o;
 	L.startt = L.t = L.t_limit = L.t_word = 0.f;
 	bool eligible = true;
-	if (ds.prob) eligible = half_bits_to_float(ds.prob[pixel_index(xy, ds.res, img)]) > 0.f;
+	if (ds.prob) eligible = !(half_bits_to_float(ds.prob[pixel_index(xy, ds.res, img)]) <= 0.f);      // occupancy_sampler.cu:571 keeps a NaN probability
 	if (!eligible) { count_finish(L, A); return; }
 	ray_through(xform, xy[0], xy[1], ds.res, ds.focal, ds.pp, &L.o, &L.d);
 	float tmin, tmax;
@@ -1287,9 +1287,9 @@ SRF_HD void loss_backward_body(uint32_t i, const LossConst& K, uint32_t n_active
 		const float weight = alpha * T;
 		r2 += weight * cr; g2 += weight * cg; b2 += weight * cb;
 		T *= (1.f - alpha);
-		const float d0 = K.loss_scale * ((weight * gr[0]) * act_rgb_derivative(raw0, K.rgb_act) + srf_max(0.0f, l2_reg * raw0));
-		const float d1 = K.loss_scale * ((weight * gr[1]) * act_rgb_derivative(raw1, K.rgb_act) + srf_max(0.0f, l2_reg * raw1));
-		const float d2 = K.loss_scale * ((weight * gr[2]) * act_rgb_derivative(raw2, K.rgb_act) + srf_max(0.0f, l2_reg * raw2));
+		const float d0 = K.loss_scale * ((weight * gr[0]) * act_rgb_derivative(raw0, K.rgb_act) + srf_max_zero(l2_reg * raw0));
+		const float d1 = K.loss_scale * ((weight * gr[1]) * act_rgb_derivative(raw1, K.rgb_act) + srf_max_zero(l2_reg * raw1));
+		const float d2 = K.loss_scale * ((weight * gr[2]) * act_rgb_derivative(raw2, K.rgb_act) + srf_max_zero(l2_reg * raw2));
 		const float sx = f.rgb_ray[0] - r2, sy = f.rgb_ray[1] - g2, sz = f.rgb_ray[2] - b2;
 		const float dd = act_density_derivative(raw3, K.density_act);
 		const float dotv = (gr[0] * (T * cr - sx) + gr[1] * (T * cg - sy)) + gr[2] * (T * cb - sz);

@@ -558,9 +558,9 @@ SRF_HD void phase_c(uint32_t tid, uint32_t win, const Args& A, const Window<G>& 
 		const float cr = act_rgb(v[0], rgb_act), cg = act_rgb(v[1], rgb_act), cb = act_rgb(v[2], rgb_act);
 		const float weight = st.alpha[j] * T_before;
 		const float T = T_before * (1.f - st.alpha[j]);          // the chain's own update (ray_marcher.cu:181)
-		const float d0 = A.K.loss_scale * ((weight * og.x) * act_rgb_derivative(v[0], rgb_act) + srf_max(0.0f, l2_reg * v[0]));
-		const float d1 = A.K.loss_scale * ((weight * og.y) * act_rgb_derivative(v[1], rgb_act) + srf_max(0.0f, l2_reg * v[1]));
-		const float d2 = A.K.loss_scale * ((weight * og.z) * act_rgb_derivative(v[2], rgb_act) + srf_max(0.0f, l2_reg * v[2]));
+		const float d0 = A.K.loss_scale * ((weight * og.x) * act_rgb_derivative(v[0], rgb_act) + srf_max_zero(l2_reg * v[0]));
+		const float d1 = A.K.loss_scale * ((weight * og.y) * act_rgb_derivative(v[1], rgb_act) + srf_max_zero(l2_reg * v[1]));
+		const float d2 = A.K.loss_scale * ((weight * og.z) * act_rgb_derivative(v[2], rgb_act) + srf_max_zero(l2_reg * v[2]));
 		const float sx = oc.x - after.y, sy = oc.y - after.z, sz = oc.z - after.w;
 		const float dd = act_density_derivative(v[3], density_act);
 		const float dotv = (og.x * (T * cr - sx) + og.y * (T * cg - sy)) + og.z * (T * cb - sz);

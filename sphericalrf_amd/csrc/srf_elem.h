@@ -36,6 +36,9 @@ SRF_HD float srf_copysign(float m, float s) { return __builtin_copysignf(m, s); 
 // fminf/fmaxf semantics of C (a NaN operand yields the other operand).
 SRF_HD float srf_min(float a, float b) { return __builtin_fminf(a, b); }
 SRF_HD float srf_max(float a, float b) { return __builtin_fmaxf(a, b); }
+// max(0, x) with +0 for either zero and for NaN.  fmaxf leaves the sign of max(+0, -0) open (host libraries and GPU
+// instructions differ); CUDA's, which the reference's fmaxf(0.0f, x) goes through, orders -0 below +0.
+SRF_HD float srf_max_zero(float x) { return x > 0.0f ? x : 0.0f; }
 
 // float -> int32 with truncation toward zero; NaN -> 0 and saturation at the
 // int32 range (what a GPU convert instruction does; a bare C cast is undefined

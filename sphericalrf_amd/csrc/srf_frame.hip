@@ -17,6 +17,15 @@ __global__ void __launch_bounds__(256) k_tonemap(uint32_t n_pixels, TonemapArgs 
 	if (i < n_pixels) out[i] = tonemap_body(acc[i], A);
 }
 
+// stand-in for the network's input gradient: a second table row, centred on zero, replaces the sample's position
+__global__ void __launch_bounds__(256) k_field_input_gradient(Params P, uint32_t n, float* __restrict__ coords, FieldArgs F) {
+	const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+	if (i >= n) return;
+	float* c = coords + 7 * (size_t)i;
+	const Float4 row = *(const Float4*)(F.table + 4 * (size_t)field_row(P, ld3(c), F));
+	c[0] = row.x - 0.5f; c[1] = row.y - 0.5f; c[2] = row.z - 0.5f;
+}
+
 } // namespace srf
 
 using namespace srf;
@@ -29,12 +38,28 @@ int srf_field_inference(void* user, uint32_t n_elements, const float* coords, vo
 	return srf_field_eval(c->sampler, c->field, n_elements, coords, rgbsigma, dtype, padded_output_width, stream);
 }
 
+int srf_field_input_gradient(void* user, uint32_t n_elements, float* coords, void* stream) {
+	const srf_field_inference_ctx* c = (const srf_field_inference_ctx*)user;
+	SRF_REQUIRE(c && c->sampler && c->field && c->field->table, "srf_field_input_gradient: NULL context");
+	SRF_REQUIRE(c->field->table_size && !(c->field->table_size & (c->field->table_size - 1)), "srf_field_input_gradient: table_size must be a power of two");
+	SRF_REQUIRE(c->sampler->P.griddist_type == SRF_GRID_WARPED_EXP || c->sampler->P.griddist_type == SRF_GRID_WARPED_RECIPROCAL, "srf_field_input_gradient: needs a warped-space grid type");
+	if (n_elements == 0) return SRF_OK;
+	SRF_REQUIRE(coords, "srf_field_input_gradient: NULL buffer");
+	const FieldArgs F{c->field->table, c->field->table_size - 1, c->field->seed ^ 0x9e3779b9u};
+	hipLaunchKernelGGL(k_field_input_gradient, dim3(div_up(n_elements, 256)), dim3(256), 0, (hipStream_t)stream, c->sampler->P, n_elements, coords, F);
+	SRF_LAUNCH_CHECK();
+	return SRF_OK;
+}
+
 int srf_render_frame(srf_sampler_t* s, srf_marcher_t* m, const srf_frame_args* a, srf_inference_fn inference, void* user,
                      float* frame_buffer, uint32_t* n_iterations, void* stream) {
 	SRF_REQUIRE(s && m && a && inference && frame_buffer, "srf_render_frame: NULL argument");
 	SRF_REQUIRE(a->resolution[0] > 0 && a->resolution[1] > 0, "srf_render_frame: resolution must be positive");
 	SRF_REQUIRE(a->padded_output_width >= 4, "srf_render_frame: padded_output_width must be >= 4");
 	SRF_REQUIRE(a->network_output_dtype == SRF_DTYPE_F16 || a->network_output_dtype == SRF_DTYPE_F32, "srf_render_frame: unknown dtype");
+	SRF_REQUIRE(a->render_mode >= SRF_RENDER_AO && a->render_mode <= SRF_RENDER_COST, "srf_render_frame: unknown render mode");
+	if (a->render_mode == SRF_RENDER_NORMALS && !a->input_gradient)
+		SRF_FAIL(SRF_ERR_UNSUPPORTED, "srf_render_frame: Normals mode composites the density's input gradient (internal/testbed.cu:558-560); args->input_gradient must supply it");
 	hipStream_t st = (hipStream_t)stream;
 	const uint32_t n_pixels = (uint32_t)a->resolution[0] * (uint32_t)a->resolution[1];
 	constexpr uint32_t MIN_STEPS = 1, MAX_STEPS = 8, MARCH_ITER = 10000;       // testbed.h: MIN/MAX_STEPS_INBETWEEN_COMPACTION, MARCH_ITER
@@ -114,6 +139,10 @@ int srf_render_frame(srf_sampler_t* s, srf_marcher_t* m, const srf_frame_args* a
 		if (rc != SRF_OK) return rc;
 		rc = inference(user, n_alive * n_steps, coords, rgbsigma, a->network_output_dtype, a->padded_output_width, st);
 		if (rc != SRF_OK) { if (rc > 0) SRF_FAIL(SRF_ERR_INVALID, "srf_render_frame: the inference callback returned %d", rc); return rc; }
+		if (a->render_mode == SRF_RENDER_NORMALS) {       // testbed.cu:558-560
+			rc = a->input_gradient(a->input_gradient_user, n_alive * n_steps, coords, st);
+			if (rc != SRF_OK) { if (rc > 0) SRF_FAIL(SRF_ERR_INVALID, "srf_render_frame: the input gradient callback returned %d", rc); return rc; }
+		}
 		ra.n_rays = n_alive; ra.n_steps = n_steps; ra.i_steps_offset = offset;
 		rc = srf_marcher_volume_rendering(m, s, &ra, pay[cur], col[cur], coords, rgbsigma, st);
 		if (rc != SRF_OK) return rc;

@@ -631,6 +631,15 @@ int srf_sampler_set_density_grid(srf_sampler_t* s, const float* density_grid, vo
 	return SRF_OK;
 }
 
+int srf_sampler_load_density_grid(srf_sampler_t* s, const float* density_grid_host, uint32_t n_values, void* stream) {
+	SRF_REQUIRE(s && density_grid_host, "srf_sampler_load_density_grid: NULL argument");
+	SRF_REQUIRE(s->P.use_grid, "srf_sampler_load_density_grid: sampler has no grid");
+	SRF_REQUIRE(n_values == s->n_total, "srf_sampler_load_density_grid: the snapshot's grid holds %u values, the configured grid has %u cells", n_values, s->n_total);
+	SRF_HIP(hipMemcpyAsync(s->density_grid, density_grid_host, (size_t)s->n_total * sizeof(float), hipMemcpyHostToDevice, (hipStream_t)stream));
+	SRF_HIP(hipStreamSynchronize((hipStream_t)stream));
+	return srf_sampler_update_grid_bitfield(s, stream);
+}
+
 int srf_sampler_set_grid_sample_order(srf_sampler_t* s, int32_t cell_order) {
 	SRF_REQUIRE(s, "srf_sampler_set_grid_sample_order: NULL sampler");
 	SRF_REQUIRE(cell_order == 0 || cell_order == 1, "srf_sampler_set_grid_sample_order: order must be 0 or 1");

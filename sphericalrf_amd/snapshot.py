@@ -34,9 +34,13 @@ def read_snapshot(path):
         raise SnapshotError("snapshot.density_grid: a binary of float32 values expected")
     if "samlper" not in cfg:
         raise SnapshotError('the snapshot holds no "samlper" block')
-    offset = snap.get("scene_offset", [0.0, 0.0, 0.0])
+    if "scene_scale" not in snap or "scene_offset" not in snap:    # testbed.cu:163-164 reads both unconditionally and throws without them
+        raise SnapshotError("snapshot.scene_scale and snapshot.scene_offset are required")
+    offset = snap["scene_offset"]
+    if not isinstance(offset, (list, tuple)) or len(offset) != 3:
+        raise SnapshotError("snapshot.scene_offset: an array of three numbers expected")
     return dict(sampler=cfg["samlper"], render=cfg.get("render", {}), loss=cfg.get("loss"),
-                density_grid=np.frombuffer(bytes(grid), dtype="<f4").copy(), scene_scale=float(snap.get("scene_scale", 1.0)),
+                density_grid=np.frombuffer(bytes(grid), dtype="<f4").copy(), scene_scale=float(snap["scene_scale"]),
                 scene_offset=tuple(float(v) for v in offset))
 
 

@@ -128,7 +128,7 @@ def test_grid_maintenance(gpu, orc, N, C, large_batch_path, monkeypatch):
 # splat of small or, forced, of large batches).  Step 2: fewer points than cells (nothing is in cell order).  Step 3: arrays handed to update_grid in
 # the reference's order although the sampler drew them in cell order (every entry fails its check; the grid is still right).
 @pytest.mark.parametrize("large_batch_path", ["0", "1"])
-@pytest.mark.parametrize("N,C", [((64, 32, 32), 5), ((128, 128, 128), 2), ((32, 32, 32), 9)])     # nine cascades: too many for update_grid's per-cell splat
+@pytest.mark.parametrize("N,C", [((64, 32, 32), 5), ((128, 128, 128), 2), ((32, 32, 32), 8), ((32, 32, 32), 9)])     # eight cascades: the most (and the most shared memory, 64 KiB) that update_grid's per-cell splat takes; nine: too many for it
 def test_grid_samples_in_cell_order(gpu, orc, N, C, large_batch_path, monkeypatch):
     torch = gpu
     monkeypatch.setenv("SRF_SPLAT_SORT", large_batch_path)
@@ -206,6 +206,8 @@ def test_training_sampler(gpu, orc, config_id, scale, budget, monkeypatch):
     rng = np.random.default_rng(config_id)
     images = rng.random((n_img * res[0] * res[1], 4)).astype(np.float16)
     prob = (rng.random(n_img * res[0] * res[1]) > 0.02).astype(np.float16)
+    prob[rng.random(prob.size) < 0.02] = np.nan         # not <= 0: such a pixel's rays are kept (occupancy_sampler.cu:571)
+    prob[rng.random(prob.size) < 0.02] = -1.0
     o_ds = orc.make_dataset(w["cameras"], res, w["focal"], (0.5, 0.5), images=images, sampling_probability=prob)
     g_ds = api.Dataset(torch.from_numpy(w["cameras"]).cuda(), res, w["focal"], (0.5, 0.5), torch.from_numpy(images).cuda(), torch.from_numpy(prob).cuda())
     n_rays = 20000
@@ -763,6 +765,57 @@ def test_library_side_frame_loop(gpu, orc, config_id, scale, inference):
     assert (want_frame[..., 3] > 0).mean() > 0.05
 
 
+@pytest.mark.parametrize("mode", ["AO", "NORMALS", "DEPTH", "DISTANCE", "COST"])
+def test_library_side_frame_loop_in_every_render_mode(gpu, orc, mode):
+    """srf_render_frame in the other render modes (internal/testbed.cu:558-560 and :603-611): Normals mode overwrites a round's
+    coordinates with the network's input gradient (here the stand-in's) before they are composited"""
+    torch = gpu
+    from sphericalrf_amd import api, scene
+    w, p, grid, bf, mean = helpers.build_scene(orc, 1, 0.25)
+    s = make_sampler(torch, api, w, grid)
+    m = api.RayMarcher(dict(train_in_linear_color=False, transmittance_threshold=1e-4))
+    res, f, cam = w["resolution"], w["focal"], w["cameras"][-1]
+    table = scene.field_table(4096, 5)
+    table[:, 3] *= 20
+    render_mode = getattr(api, "RENDER_" + mode)
+    want_frame, _, iters = orc.render_frame(p, orc.make_field(table, 77), bf, res, f, (0.5, 0.5), cam, transmittance_threshold=1e-4, train_in_linear_colors=False,
+                                            render_mode=render_mode)
+    shade_frame, _, _ = orc.render_frame(p, orc.make_field(table, 77), bf, res, f, (0.5, 0.5), cam, transmittance_threshold=1e-4, train_in_linear_colors=False)
+    assert not np.array_equal(want_frame, shade_frame)
+    field = api.Field(torch.from_numpy(table).cuda(), 77)
+    frame = torch.ones((res[1], res[0], 4), device="cuda")
+    got_iters = s.render_frame(m, field, res, f, (0.5, 0.5), cam, frame, render_mode=render_mode, density_activation=api.ACT_NONE, rgb_activation=api.ACT_NONE,
+                               network_output_dtype=api.DTYPE_F32, input_gradient=True if mode == "NORMALS" else None)
+    assert got_iters == iters and np.array_equal(frame.cpu().numpy(), want_frame)
+    if mode == "NORMALS":
+        # without the gradient step the positions themselves would be composited: a different frame, so the mode is refused
+        with pytest.raises(api.SrfError) as e:
+            s.render_frame(m, field, res, f, (0.5, 0.5), cam, frame, render_mode=render_mode, density_activation=api.ACT_NONE, rgb_activation=api.ACT_NONE,
+                           network_output_dtype=api.DTYPE_F32)
+        assert e.value.code == api.ERR_UNSUPPORTED
+
+
+def test_an_exception_in_the_inference_callback_ends_the_frame(gpu, orc):
+    """a Python network that raises: srf_render_frame stops at that round and the exception reaches the caller"""
+    torch = gpu
+    from sphericalrf_amd import api
+    w, p, grid, bf, mean = helpers.build_scene(orc, 1, 0.25)
+    s = make_sampler(torch, api, w, grid)
+    m = api.RayMarcher(dict(train_in_linear_color=False))
+    res, f, cam = w["resolution"], w["focal"], w["cameras"][-1]
+    calls = []
+
+    def net(n_elements, coords, out, dtype, width, stream):
+        calls.append(n_elements)
+        raise KeyError("no such layer")
+
+    frame = torch.ones((res[1], res[0], 4), device="cuda")
+    with pytest.raises(KeyError):
+        s.render_frame(m, net, res, f, (0.5, 0.5), cam, frame)
+    torch.cuda.synchronize()
+    assert len(calls) == 1
+
+
 @pytest.mark.parametrize("color_space", [0, 1, 2])
 def test_accumulate_and_tonemap(gpu, orc, color_space):
     """CudaRenderBuffer::accumulate and ::tonemap (internal/utils/render_buffer.cu:46-178): four frames into the running mean, then every
@@ -876,6 +929,35 @@ def test_render_modes_and_half_network_output(gpu, orc):
             assert np.array_equal(d_rgba.cpu().numpy(), o_rgba, equal_nan=True), (mode, dtype)
 
 
+@pytest.mark.parametrize("train_in_linear", [False, True])
+@pytest.mark.parametrize("mode", ["SHADE", "NORMALS", "COST", "DEPTH"])
+def test_shade_in_every_branch(gpu, orc, mode, train_in_linear):
+    """shade_kernel (internal/testbed.cu:448-477) on its own: normals remapped to colours, the step count of Cost mode, the
+    sRGB-to-linear conversion of a frame trained in sRGB, blended over a frame buffer that is not empty"""
+    torch = gpu
+    from sphericalrf_amd import api
+    rng = np.random.default_rng(len(mode) + 10 * train_in_linear)
+    res = (53, 31)
+    n_pixels = res[0] * res[1]
+    n = n_pixels - 100
+    pay = np.zeros(n, O.PAYLOAD_DTYPE)
+    pay["idx"] = rng.permutation(n_pixels)[:n]
+    pay["n_steps"] = rng.integers(0, 400, n)
+    rgba = rng.random((n, 4)).astype(np.float32)
+    if mode == "NORMALS":
+        rgba[:, :3] = rgba[:, :3] * 2 - 1
+        rgba[:7, :3] = 0            # a zero normal: normalised to NaN by the reference as well
+    frame0 = (rng.random((n_pixels, 4)) * 0.5).astype(np.float32)
+    want = frame0.copy()
+    render_mode = getattr(O, "RENDER_" + mode)
+    orc.shade(n, rgba, pay, want, render_mode, train_in_linear)
+    fb = torch.from_numpy(frame0).cuda()
+    api.shade(n, torch.from_numpy(rgba).cuda(), torch.from_numpy(pay.view(np.uint8)).cuda(), fb, render_mode, train_in_linear)
+    got = fb.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)) or np.array_equal(got, want, equal_nan=True)
+    assert not np.array_equal(want, frame0, equal_nan=True)
+
+
 def test_rollover_fill(gpu, orc):
     torch = gpu
     from sphericalrf_amd import api
@@ -918,14 +1000,15 @@ def test_errors_are_reported_not_thrown_across_the_abi(gpu):
 
 
 @pytest.mark.parametrize("impl", ["waves", "stream"])
-@pytest.mark.parametrize("acts", ["plain", "activated"])
+@pytest.mark.parametrize("acts", ["plain", "activated", "relu"])
 @pytest.mark.parametrize("kind", ["short", "long", "split", "tiny", "gaps", "biggap", "shuffled"])
 def test_single_launch_compositing_layouts(gpu, orc, kind, acts, impl, monkeypatch):
     """every sample layout the streaming compositing distinguishes (back-to-back rays, holes, groups longer than a window,
     shuffled offsets), against the oracle, over many workgroups so that its ordered offsets really go through the chain;
-    with the activations compiled out ("plain": both None) and with the run-time switches (Logistic colour, Exponential density)"""
+    with the activations compiled out ("plain": both None) and with the run-time switches (Logistic colour and Exponential density;
+    ReLU for both, over outputs of either sign)"""
     monkeypatch.setenv("SRF_COMPOSITE_IMPL", impl)
-    rgb_act, den_act = (O.ACT_NONE, O.ACT_NONE) if acts == "plain" else (O.ACT_LOGISTIC, O.ACT_EXPONENTIAL)
+    rgb_act, den_act = {"plain": (O.ACT_NONE, O.ACT_NONE), "activated": (O.ACT_LOGISTIC, O.ACT_EXPONENTIAL), "relu": (O.ACT_RELU, O.ACT_RELU)}[acts]
     torch = gpu
     from sphericalrf_amd import api
     from tests.test_fused_compositing_on_host import layout
@@ -936,6 +1019,9 @@ def test_single_launch_compositing_layouts(gpu, orc, kind, acts, impl, monkeypat
     net[:, 3] *= np.float16(0.05 if kind == "long" else 3)
     if acts == "activated":
         net[:, 3] = np.log(net[:, 3].astype(np.float32) + 1e-3).astype(np.float16)      # the exponential brings the densities back
+    if acts == "relu":
+        net[:, :3] -= np.float16(0.3)          # a third of the colours and of the densities below zero: clamped, with zero derivative
+        net[:, 3] -= np.float16(0.4 * (0.05 if kind == "long" else 3))
     dt = (rng.random(total) * 0.3 + 0.01).astype(np.float32)
     tgt = rng.random((n_rays, 4)).astype(np.float32)
     cap = int(counts.sum() * 0.9) + 1
@@ -968,7 +1054,7 @@ def test_single_launch_compositing_layouts(gpu, orc, kind, acts, impl, monkeypat
 def test_a_look_back_that_gives_up_is_reported_and_the_marcher_falls_back(gpu, orc, monkeypatch):
     """With no polls allowed, an item of the streaming compositing whose predecessors' counts are not there at its first look
     gives up (the kernel still drains normally).  The call's counter then reads 0xffffffff, the failure is returned by
-    sync_check, and the marcher's later calls take the three-launch implementation and are right again.  (If every first look
+    sync_check, and the marcher's later calls take the wave-per-item kernel and are right again.  (If every first look
     succeeds, nothing gives up, and the results must simply be right.)"""
     monkeypatch.delenv("SRF_COMPOSITE_IMPL", raising=False)
     torch = gpu
@@ -1006,7 +1092,7 @@ def test_a_look_back_that_gives_up_is_reported_and_the_marcher_falls_back(gpu, o
         assert "gave up" in str(e)
         assert int(cnt.item()) & 0xffffffff == 0xffffffff
     if gave_up:
-        d_idx, d_dloss, cnt = call()      # the three-launch implementation from here on
+        d_idx, d_dloss, cnt = call()      # the wave-per-item kernel from here on
         m.sync_check()
     assert int(cnt.item()) == o_total and np.array_equal(u32(d_idx), o_idx)
     assert np.array_equal(d_dloss.cpu().numpy().view(np.uint32), o_dloss.view(np.uint32))

@@ -38,6 +38,8 @@ MUTATIONS = [
      pins.pin_sampling_probability_pixel, "occupancy_sampler.cu:569"),
     ("probability_test_sign", "if (half_to_float(ds->sampling_probability[pidx]) <= 0.f) continue;", "if (half_to_float(ds->sampling_probability[pidx]) > 0.f) continue;",
      pins.pin_sampling_probability_pixel, "occupancy_sampler.cu:570"),
+    ("nan_probability_skipped", "if (half_to_float(ds->sampling_probability[pidx]) <= 0.f) continue;", "if (!(half_to_float(ds->sampling_probability[pidx]) > 0.f)) continue;",
+     pins.pin_sampling_probability_pixel, "occupancy_sampler.cu:571"),
     ("snap_without_half_pixel", "xy[a] = ((float)px + 0.5f) / (float)res[a];", "xy[a] = ((float)px) / (float)res[a];",
      pins.pin_training_rays, "occupancy_sampler.cu:566"),
     ("snap_always", "if (P.snap_to_pixel_centers_in_training) {", "if (true) {",

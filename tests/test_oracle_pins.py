@@ -120,7 +120,8 @@ def pin_training_rays_without_snapping(orc):
 
 
 def pin_sampling_probability_pixel(orc):
-    """a ray is skipped exactly when the probability AT ITS OWN PIXEL (x + y*W + img*W*H) is <= 0 (:569-570)"""
+    """a ray is skipped exactly when the probability AT ITS OWN PIXEL (x + y*W + img*W*H) is <= 0 (:569-570); a negative one skips
+    it too, and a NaN, which is not <= 0, keeps it"""
     p, cams, res, focal, pp, images = _training_case(orc, 64, 0.5, 0.3)
     n_rays, seed = 60, 21
     expected = [_expected_training_ray(orc, p, cams, res, focal, pp, seed, i, n_rays, 0, snap=1) for i in range(n_rays)]
@@ -128,10 +129,13 @@ def pin_sampling_probability_pixel(orc):
     zeroed = set(hit[::2])                                          # every second pixel that some ray lands on
     prob = np.ones(cams.shape[0] * res[0] * res[1], np.float16)
     prob[list(zeroed)] = 0
+    prob[hit[2]] = -0.5
+    prob[hit[1]] = np.nan
     ds = orc.make_dataset(cams, res, focal, pp, images=images, sampling_probability=prob)
     bf = np.full(p.n_total // 8, 0xff, np.uint8)
     out = orc.generate_training_samples(p, n_rays, 0, 1 << 16, ds, bf, orc.pcg32(seed))
     kept = [i for i, e in enumerate(expected) if e["pixel_index"] not in zeroed]
+    assert any(e["pixel_index"] == hit[1] for e in expected)
     assert 0 < len(kept) < n_rays
     assert out["ray_counter"] == len(kept)
     assert np.array_equal(out["src"][:len(kept)], np.uint32(kept))

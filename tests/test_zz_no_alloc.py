@@ -24,21 +24,26 @@ def _inputs(torch, seed, n_rays, kind):
     return dict(n_rays=n_rays, total=total, cap=cap, idx=idx, net=dev(net), dt=dev(dt), tgt=dev(tgt), coords=dev(coords))
 
 
-def _run(torch, api, marcher, w, no_alloc):
+def _buffers(torch, w):
     n_rays, cap = w["n_rays"], w["cap"]
-    idx = torch.from_numpy(w["idx"].view(np.int32)).cuda()
-    dloss = torch.zeros((cap, 4), device="cuda")
-    compacted = torch.zeros((cap, 7), device="cuda")
-    loss, rgb = torch.full((n_rays,), -1.0, device="cuda"), torch.zeros((n_rays, 3), device="cuda")
-    cnt = torch.full((1,), 5, dtype=torch.int32, device="cuda")
-    nrc = torch.full((1,), n_rays - 3, dtype=torch.int32, device="cuda")
-    mean_t = torch.full((1,), 0.001, device="cuda")
-    marcher.volume_rendering_with_loss_and_gradient(n_rays, cap, w["tgt"], nrc, idx, w["dt"], w["net"], dloss, cnt, rgb_activation=api.ACT_LOGISTIC,
-                                                    density_activation=api.ACT_EXPONENTIAL, loss_output=loss, loss_type="SMAPE", density_grid_mean=mean_t,
-                                                    use_grid=True, background_color=(0.2, 0.4, 0.6), coords=w["coords"], compacted_coords=compacted,
-                                                    rgb_ray_out=rgb, no_alloc=no_alloc)
+    return dict(idx=torch.from_numpy(w["idx"].view(np.int32)).cuda(), dloss=torch.zeros((cap, 4), device="cuda"), compacted=torch.zeros((cap, 7), device="cuda"),
+                loss=torch.full((n_rays,), -1.0, device="cuda"), rgb=torch.zeros((n_rays, 3), device="cuda"),
+                cnt=torch.full((1,), 5, dtype=torch.int32, device="cuda"), nrc=torch.full((1,), n_rays - 3, dtype=torch.int32, device="cuda"),
+                mean=torch.full((1,), 0.001, device="cuda"))
+
+
+def _call(api, marcher, w, b, no_alloc):
+    marcher.volume_rendering_with_loss_and_gradient(w["n_rays"], w["cap"], w["tgt"], b["nrc"], b["idx"], w["dt"], w["net"], b["dloss"], b["cnt"], rgb_activation=api.ACT_LOGISTIC,
+                                                    density_activation=api.ACT_EXPONENTIAL, loss_output=b["loss"], loss_type="SMAPE", density_grid_mean=b["mean"],
+                                                    use_grid=True, background_color=(0.2, 0.4, 0.6), coords=w["coords"], compacted_coords=b["compacted"],
+                                                    rgb_ray_out=b["rgb"], no_alloc=no_alloc)
     marcher.sync_check()
-    return [t.cpu().numpy().view(np.uint32) for t in (cnt, idx, dloss, compacted, loss, rgb)]
+
+
+def _run(torch, api, marcher, w, no_alloc):
+    b = _buffers(torch, w)
+    _call(api, marcher, w, b, no_alloc)
+    return [b[k].cpu().numpy().view(np.uint32) for k in ("cnt", "idx", "dloss", "compacted", "loss", "rgb")]
 
 
 def test_no_alloc_entry_point_matches_the_ordinary_one_twice_in_a_row(gpu, monkeypatch):
@@ -55,6 +60,29 @@ def test_no_alloc_entry_point_matches_the_ordinary_one_twice_in_a_row(gpu, monke
         assert int(want[0][0]) > 5
         for x, y in zip(want, got):
             assert np.array_equal(x, y)
+
+
+def test_no_alloc_entry_point_leaves_the_free_device_memory_alone(gpu, monkeypatch):
+    """After one call per device (which looks up the scratch symbol and the kernel's occupancy), a call with more rays than any
+    before changes the device's free memory by nothing, where the ordinary entry point's growing workspace is seen to."""
+    torch = gpu
+    from sphericalrf_amd import api
+    monkeypatch.delenv("SRF_COMPOSITE_IMPL", raising=False)
+    cfg = dict(train_with_random_bg_color=True, train_in_linear_color=False)
+    no_alloc, ordinary = api.RayMarcher(cfg), api.RayMarcher(cfg)
+    small, large = _inputs(torch, 43, 64 * 30, "short"), _inputs(torch, 44, 64 * 4000 + 3, "short")
+    b_small, b_large = _buffers(torch, small), _buffers(torch, large)
+    _call(api, no_alloc, small, b_small, True)
+    _call(api, ordinary, small, b_small, False)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    _call(api, no_alloc, large, b_large, True)
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    assert free_after == free_before
+    _call(api, ordinary, large, b_large, False)       # the control: this one has to grow its workspace (about 19 bytes a ray)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] < free_after
 
 
 def test_no_alloc_entry_point_rejects_what_it_cannot_serve(gpu, monkeypatch):
