@@ -8,9 +8,13 @@ timed region.  The one JSON line printed on stdout carries the headline metric (
 steps), the roofline of the compositing kernels (the HBM-bound part the path is specified against) and a CPU baseline:
 the oracle timed on this machine's host cores on a bounded slice of the same workload.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
 
---all adds the other four workloads (renders of workloads 1-3 and 5, grid maintenance of workload 5) under "extras".
+Under "extras" the same line carries the other workloads, each with a roofline block of its own from its algorithmic bytes: one
+frame each of workloads 1, 2, 3 and 5 (fused kernel, and the reference's loop of entry points), workload 5's grid update in both
+point orders (the draw of the first 256 steps and the steady-state draw), workload 4 in drop-in mode (Coordinate records written by
+the march and compacted by the compositing, as the reference's caller needs them) and workload 4 on a grid with about 15 % of its
+bits set, where the batch wants far more than the 2^24 samples there is room for.  --no-extras leaves them out.
 """
 import argparse
 import json
@@ -34,6 +38,15 @@ MARCH_BYTES_PER_RAY = 32         # read ray 24, write (count, offset) 8
 COMPOSITE_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "compositing_config4_hbm_traffic.txt")
 EMA_BYTES_PER_CELL = 12
 BITFIELD_BYTES_PER_CELL = 4.125
+RENDER_BYTES_PER_SAMPLE = 20     # forward-only compositing: read fp32 rgb-sigma 16 + fp32 dt 4
+RENDER_BYTES_PER_RAY = 16        # write RGBA
+COORD_BYTES = 28                 # one Coordinate record (drop-in mode: written by the march, read and written again by the compositing)
+
+
+def roofline(kernel, n_bytes, seconds):
+    gbs = n_bytes / seconds / 1e9
+    return {"kernel": kernel, "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+            "algorithmic_bytes": n_bytes}
 
 
 def composite_traffic_bytes():
@@ -71,8 +84,12 @@ def timed(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 << 24):
+def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 << 24, drop_in=False, shell=None):
+    """drop_in: the march also writes the reference's Coordinate records and the compositing copies those of the samples it keeps
+    (what Testbed::train hands to the network and its backward pass); shell: replaces the workload's shell (lo, hi, coverage)"""
     w = scene.workload(4)
+    if shell is not None:
+        w = dict(w, shell=shell)
     t0 = time.perf_counter()
     s, grid = build_sampler(torch, api, scene, w)
     log("scene built in %.1f s" % (time.perf_counter() - t0))
@@ -89,6 +106,8 @@ def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 
     sample_t = torch.zeros(cap, device=dev)
     sample_dt = torch.zeros(cap, device=dev)
     sample_cell = torch.zeros(cap, dtype=torch.int32, device=dev)
+    coords = torch.zeros((cap, 7), device=dev) if drop_in else None
+    compacted_coords = torch.zeros((cap, 7), device=dev) if drop_in else None
     n_rays_counter = torch.zeros(1, dtype=torch.int32, device=dev)
     n_coords_counter = torch.zeros(1, dtype=torch.int32, device=dev)
     n_compacted = torch.zeros(1, dtype=torch.int32, device=dev)
@@ -106,6 +125,7 @@ def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
     times = {"march": [], "composite": []}
     state = {"shift": 0}
+    rng_last = [None]           # the generator as the last step's march saw it
 
     def step(record=False):
         n_rays_counter.zero_()
@@ -113,19 +133,22 @@ def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 
         n_compacted.zero_()
         if record:
             ev[0].record()
-        s.sample_coords_from_dataset(n_rays, state["shift"], cap, ds, rays, rays_rgba, n_rays_counter, ray_idx, None, n_coords_counter, rng,
+        s.sample_coords_from_dataset(n_rays, state["shift"], cap, ds, rays, rays_rgba, n_rays_counter, ray_idx, coords, n_coords_counter, rng,
                                      sample_t, sample_dt, sample_cell)
         if record:
             ev[1].record()
         m.volume_rendering_with_loss_and_gradient(n_rays, cap, targets, n_rays_counter, ray_idx, sample_dt, net, dloss, n_compacted,
                                                   rgb_activation=api.ACT_NONE, density_activation=api.ACT_NONE, loss_output=loss, loss_type="L2",
-                                                  loss_scale=128.0, density_grid_mean=s.density_grid_mean, use_grid=True, dt_stride=1, rgb_ray_out=rgb_out)
+                                                  loss_scale=128.0, density_grid_mean=s.density_grid_mean, use_grid=True, dt_stride=1, rgb_ray_out=rgb_out,
+                                                  coords=coords, compacted_coords=compacted_coords)
         if record:
             ev[2].record()
             torch.cuda.synchronize()
             times["march"].append(ev[0].elapsed_time(ev[1]))
             times["composite"].append(ev[1].elapsed_time(ev[2]))
         state["shift"] += n_rays
+        rng_last[0] = api.Pcg32(0)
+        rng_last[0].state, rng_last[0].inc = rng.state, rng.inc
         rng.advance()
 
     step()
@@ -136,13 +159,25 @@ def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 
     # per-part times over separate instrumented steps (event records around each entry point, on the stream they run on)
     for _ in range(max(3, min(steps, 10))):
         step(record=True)
-    n_kept, n_samples, n_comp = int(n_rays_counter.item()), int(n_coords_counter.item()) & 0xffffffff, int(n_compacted.item()) & 0xffffffff
+    n_kept, n_wanted, n_comp = int(n_rays_counter.item()), int(n_coords_counter.item()) & 0xffffffff, int(n_compacted.item()) & 0xffffffff
+    # the samples of the rays that were kept: the counter itself keeps growing past the capacity (occupancy_sampler.cu:638-642)
+    # (read after a march on its own: the compositing overwrites the per-ray counts with the compacted ones)
+    n_rays_counter.zero_()
+    n_coords_counter.zero_()
+    state["shift"] -= n_rays
+    s.sample_coords_from_dataset(n_rays, state["shift"], cap, ds, rays, rays_rgba, n_rays_counter, ray_idx, coords, n_coords_counter, rng_last[0],
+                                 sample_t, sample_dt, sample_cell)
+    n_samples = int(ray_idx[:n_kept, 0].long().sum().item())
     march_ms = sum(times["march"]) / len(times["march"])
     comp_ms = sum(times["composite"]) / len(times["composite"])
     comp_bytes = COMPOSITE_BYTES_PER_SAMPLE * n_samples + COMPOSITE_BYTES_PER_RAY * n_kept
     march_bytes = MARCH_BYTES_PER_SAMPLE * n_samples + MARCH_BYTES_PER_RAY * n_rays
+    if drop_in:
+        comp_bytes += COORD_BYTES * (n_samples + n_comp)       # the kept samples' records read, the compacted ones written
+        march_bytes += COORD_BYTES * n_samples
     info = s.info
-    return dict(sec_per_step=sec, n_rays=n_rays, n_kept=n_kept, n_samples=n_samples, n_compacted=n_comp, march_ms=march_ms, composite_ms=comp_ms,
+    return dict(sec_per_step=sec, n_rays=n_rays, n_kept=n_kept, n_samples=n_samples, n_samples_wanted=n_wanted, n_compacted=n_comp, march_ms=march_ms, composite_ms=comp_ms,
+                composite_bytes=comp_bytes, march_bytes=march_bytes,
                 composite_gbs=comp_bytes / (comp_ms * 1e-3) / 1e9, march_gbs=march_bytes / (march_ms * 1e-3) / 1e9,
                 n_max_steps=int(info.n_max_steps), workload=w, sampler=s, occupied_bits=occupied_bits)
 
@@ -216,8 +251,12 @@ def bench_render(torch, api, scene, config_id, steps, warmup, n_frames=2):
     loop_sec = timed(torch, loop_step, steps, warmup)
     bits = s.density_grid_bitfield
     occ = float(torch.from_numpy(__import__("numpy").unpackbits(bits.cpu().numpy())).float().mean())
+    n_bytes = RENDER_BYTES_PER_SAMPLE * total + RENDER_BYTES_PER_RAY * n
     return dict(workload="render_%d" % config_id, resolution=list(res), ms_per_frame=sec * 1e3, rays_per_s=n / sec, composited_samples_last_frame=total,
-                samples_per_s=total / sec, loop_ms_per_frame=loop_sec * 1e3, loop_rounds_last_frame=rounds["n"], occupied_bits=occ, frames_in_workload=len(cams))
+                samples_per_s=total / sec, loop_ms_per_frame=loop_sec * 1e3, loop_rounds_last_frame=rounds["n"], occupied_bits=occ, frames_in_workload=len(cams),
+                roofline=roofline("whole frame in one kernel: march + forward compositing (bytes: what the reference's loop moves per composited sample and per ray; "
+                                  "the fused kernel itself keeps them in registers and is bound by the march's instruction issue)", n_bytes, sec),
+                loop_roofline=roofline("the same frame through srf_render_frame's rounds of compact / generate_coords / inference / volume_rendering", n_bytes, loop_sec))
 
 
 def bench_grid_update(torch, api, scene, steps, warmup, cell_order=False, steady_state=False):
@@ -262,7 +301,9 @@ def bench_grid_update(torch, api, scene, steps, warmup, cell_order=False, steady
     return dict(workload="grid_update_5" + ("_steady_state" if steady_state else "") + ("_cell_order" if cell_order else ""), cells=n_total, points=n_points,
                 ms_per_update=sec * 1e3, parts_ms=avg, occupied_bits=occ,
                 update_grid_gbs=EMA_BYTES_PER_CELL * n_total / (avg["update_grid"] * 1e-3) / 1e9,
-                bitfield_gbs=BITFIELD_BYTES_PER_CELL * n_total / (avg["update_grid_bitfield"] * 1e-3) / 1e9)
+                bitfield_gbs=BITFIELD_BYTES_PER_CELL * n_total / (avg["update_grid_bitfield"] * 1e-3) / 1e9,
+                roofline=roofline("update_grid + update_grid_bitfield (12.125 B per cell: density 4 + grid read 4 + grid write 4 + bit 1/8)",
+                                  (EMA_BYTES_PER_CELL + 0.125) * n_total, (avg["update_grid"] + avg["update_grid_bitfield"]) * 1e-3))
 
 
 def bench_grid_sample_draws(torch, api, scene, steps):
@@ -286,7 +327,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--all", action="store_true", help="also run the render and grid-maintenance workloads")
+    ap.add_argument("--no-extras", action="store_true", help="only the headline workload (the other workloads under \"extras\" take about a minute)")
+    ap.add_argument("--all", action="store_true", help="accepted for older command lines: the extras are on by default")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (read 2^30 B, write 2^30 B each) so that a counter run has a kernel of known traffic to scale by")
@@ -328,20 +370,34 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(r)
-    if args.all:
+    if not args.no_extras:
         extras = []
         del r["sampler"]
         torch.cuda.empty_cache()
+        k = max(2, args.steps // 2)
         for cid in (1, 2, 3, 5):
-            extras.append(bench_render(torch, api, scene, cid, max(2, args.steps // 2), 1))
+            extras.append(bench_render(torch, api, scene, cid, k, 1))
             log(json.dumps(extras[-1]))
             torch.cuda.empty_cache()
-        extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1))
-        extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1, cell_order=True))
-        extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1, steady_state=True))
-        extras.append(bench_grid_update(torch, api, scene, max(2, args.steps // 2), 1, cell_order=True, steady_state=True))
-        extras.append(bench_grid_sample_draws(torch, api, scene, max(2, args.steps // 2)))
+        for cell_order, steady in ((False, False), (True, False), (False, True), (True, True)):
+            extras.append(bench_grid_update(torch, api, scene, k, 1, cell_order=cell_order, steady_state=steady))
+            log(json.dumps(extras[-1]))
+        extras.append(bench_grid_sample_draws(torch, api, scene, k))
         log(json.dumps(extras[-1]))
+        torch.cuda.empty_cache()
+        for name, kw in (("training_step_4_drop_in", dict(drop_in=True)),
+                         ("training_step_4_dense_grid", dict(shell=(0.05, 1.0, 1.0)))):
+            t = bench_training_step(torch, api, scene, k, 1, **kw)
+            extras.append(dict(
+                workload=name, ms_per_step=t["sec_per_step"] * 1e3, rays=t["n_rays"], rays_kept=t["n_kept"], rays_dropped_or_empty=t["n_rays"] - t["n_kept"],
+                samples=t["n_samples"], samples_wanted=t["n_samples_wanted"], sample_cap=1 << 24, compacted_samples=t["n_compacted"], occupied_bits=t["occupied_bits"],
+                marched_samples_per_s=t["n_samples"] / t["sec_per_step"], march_ms=t["march_ms"], composite_ms=t["composite_ms"],
+                roofline=roofline("compositing forward+backward" + (" with the Coordinate records of the kept samples copied (28 B read + 28 B written each)" if kw.get("drop_in") else ""),
+                                  t["composite_bytes"], t["composite_ms"] * 1e-3),
+                march_roofline=roofline("training march (output bytes; the kernel is bound by instruction issue)", t["march_bytes"], t["march_ms"] * 1e-3)))
+            log(json.dumps(extras[-1]))
+            del t
+            torch.cuda.empty_cache()
         out["extras"] = extras
     print(json.dumps(out), flush=True)
 
