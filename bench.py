@@ -249,14 +249,24 @@ def bench_render(torch, api, scene, config_id, steps, warmup, n_frames=2):
 
     k["i"] = 0
     loop_sec = timed(torch, loop_step, steps, warmup)
+
+    def paced_step():       # the same loop with the rounds' numbers kept on the device
+        rounds["n"] = s.render_frame(m, field, res, w["focal"], (0.5, 0.5), cams[k["i"] % len(cams)], frame, density_activation=api.ACT_NONE,
+                                     rgb_activation=api.ACT_NONE, network_output_dtype=api.DTYPE_F32, paced=True)
+        k["i"] += 1
+
+    k["i"] = 0
+    paced_sec = timed(torch, paced_step, steps, warmup)
     bits = s.density_grid_bitfield
     occ = float(torch.from_numpy(__import__("numpy").unpackbits(bits.cpu().numpy())).float().mean())
     n_bytes = RENDER_BYTES_PER_SAMPLE * total + RENDER_BYTES_PER_RAY * n
     return dict(workload="render_%d" % config_id, resolution=list(res), ms_per_frame=sec * 1e3, rays_per_s=n / sec, composited_samples_last_frame=total,
-                samples_per_s=total / sec, loop_ms_per_frame=loop_sec * 1e3, loop_rounds_last_frame=rounds["n"], occupied_bits=occ, frames_in_workload=len(cams),
+                samples_per_s=total / sec, loop_ms_per_frame=loop_sec * 1e3, paced_loop_ms_per_frame=paced_sec * 1e3, loop_rounds_last_frame=rounds["n"], occupied_bits=occ,
+                frames_in_workload=len(cams),
                 roofline=roofline("whole frame in one kernel: march + forward compositing (bytes: what the reference's loop moves per composited sample and per ray; "
                                   "the fused kernel itself keeps them in registers and is bound by the march's instruction issue)", n_bytes, sec),
-                loop_roofline=roofline("the same frame through srf_render_frame's rounds of compact / generate_coords / inference / volume_rendering", n_bytes, loop_sec))
+                loop_roofline=roofline("the same frame through srf_render_frame's rounds of compact / generate_coords / inference / volume_rendering", n_bytes, loop_sec),
+                paced_loop_roofline=roofline("the same rounds with their sizes kept on the device (srf_render_frame_paced)", n_bytes, paced_sec))
 
 
 def bench_grid_update(torch, api, scene, steps, warmup, cell_order=False, steady_state=False):

@@ -321,6 +321,9 @@ int  srf_render_frame_fused(srf_sampler_t* s, const srf_marcher_t* m, const srf_
 /* the stand-in evaluated over an array of Coordinate records (what the harness calls in place of the network) */
 int  srf_field_eval(const srf_sampler_t* s, const srf_field* field, uint32_t n_coords, const float* coords,
                     void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream);
+/* the same with the number of records read from device memory when the kernel starts (*n_coords_dev <= max_coords; NULL: max_coords) */
+int  srf_field_eval_counted(const srf_sampler_t* s, const srf_field* field, const uint32_t* n_coords_dev, uint32_t max_coords, const float* coords,
+                            void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream);
 
 /* ---------------- a whole frame, library side ---------------- */
 /* What a caller's network does between srf_sampler_generate_coords_from_rays and srf_marcher_volume_rendering
@@ -363,6 +366,28 @@ int  srf_field_inference(void* user, uint32_t n_elements, const float* coords, v
 /* an srf_input_gradient_fn for the stand-in field (user as above): the position of each record becomes the first three values,
  * minus one half, of the table row that the field with seed ^ 0x9e3779b9 selects for it */
 int  srf_field_input_gradient(void* user, uint32_t n_elements, float* coords, void* stream);
+
+/*
+ * srf_render_frame with the loop paced by the device.  The reference's loop (internal/testbed.cu:526-597) learns on the host, once a
+ * round, how many rays are left, and sizes the round's launches by it; the GPU idles while the host finds out.  Here the numbers
+ * of a round (rays left, n_steps, i_steps_offset) stay in device memory: the compaction writes them, the kernels of the round read
+ * them, launched over an upper limit that the host knows (the last count it has seen arrive, which can only have fallen since).
+ * The host runs a few rounds ahead of the device and stops launching once it sees a count of zero; rounds launched past the end
+ * return at once.  The network therefore gets its element count as a device pointer plus an upper limit (at most resolution.x *
+ * resolution.y): a network that needs the count on the host cannot be used here and goes through srf_render_frame.
+ * input_gradient may be NULL except in Normals mode.  Frame and *n_iterations are those of srf_render_frame; the host waits for
+ * the stream once, at the end, and only when n_iterations is not NULL.
+ */
+typedef int (*srf_inference_counted_fn)(void* user, const uint32_t* n_elements, uint32_t max_elements, const float* coords, void* rgbsigma,
+                                        int32_t dtype, uint32_t padded_output_width, void* stream);
+typedef int (*srf_input_gradient_counted_fn)(void* user, const uint32_t* n_elements, uint32_t max_elements, float* coords, void* stream);
+int  srf_render_frame_paced(srf_sampler_t* s, srf_marcher_t* m, const srf_frame_args* args, srf_inference_counted_fn inference, void* user,
+                            srf_input_gradient_counted_fn input_gradient, void* input_gradient_user,
+                            float* frame_buffer, uint32_t* n_iterations, void* stream);
+/* the stand-in field as such callbacks (user points at an srf_field_inference_ctx) */
+int  srf_field_inference_counted(void* user, const uint32_t* n_elements, uint32_t max_elements, const float* coords, void* rgbsigma,
+                                 int32_t dtype, uint32_t padded_output_width, void* stream);
+int  srf_field_input_gradient_counted(void* user, const uint32_t* n_elements, uint32_t max_elements, float* coords, void* stream);
 
 /* CudaRenderBuffer::accumulate, internal/utils/render_buffer.cu:46-85, :211-227: running mean of the frames of one view.  spp is the
  * number of frames already accumulated (0: the buffer is cleared first); the caller counts. */

@@ -102,6 +102,9 @@ class FieldInferenceCtx(C.Structure):
 INFERENCE_FN = C.CFUNCTYPE(C.c_int, vp, u32, vp, vp, i32, u32, vp)
 # srf_input_gradient_fn: (user, n_elements, coords, stream) -> int
 INPUT_GRADIENT_FN = C.CFUNCTYPE(C.c_int, vp, u32, vp, vp)
+# the same with the element count in device memory: (user, n_elements_dev, max_elements, ...)
+INFERENCE_COUNTED_FN = C.CFUNCTYPE(C.c_int, vp, vp, u32, vp, vp, i32, u32, vp)
+INPUT_GRADIENT_COUNTED_FN = C.CFUNCTYPE(C.c_int, vp, vp, u32, vp, vp)
 
 
 # every symbol include/srf_hip.h declares
@@ -114,7 +117,8 @@ SYMBOLS = [
     "srf_marcher_config_default", "srf_marcher_create", "srf_marcher_destroy", "srf_marcher_get_config", "srf_marcher_set_config",
     "srf_marcher_volume_rendering_with_loss_and_gradient", "srf_marcher_volume_rendering_with_loss_and_gradient_noalloc", "srf_marcher_sync_check", "srf_marcher_volume_rendering",
     "srf_compact_rays", "srf_shade", "srf_fill_rollover", "srf_fill_rollover_and_rescale",
-    "srf_render_frame", "srf_field_inference", "srf_field_input_gradient", "srf_frame_accumulate", "srf_frame_tonemap",
+    "srf_render_frame", "srf_field_inference", "srf_field_input_gradient", "srf_render_frame_paced", "srf_field_inference_counted",
+    "srf_field_input_gradient_counted", "srf_field_eval_counted", "srf_frame_accumulate", "srf_frame_tonemap",
     "srf_render_frame_fused", "srf_field_eval", "srf_debug_eval_elem", "srf_marcher_debug_set_lookback_spin_limit",
 ]
 
@@ -182,6 +186,10 @@ def load():
     L.srf_render_frame.argtypes = [vp, vp, P(FrameArgs), vp, vp, vp, P(u32), vp]
     L.srf_field_inference.argtypes = [vp, u32, vp, vp, i32, u32, vp]
     L.srf_field_input_gradient.argtypes = [vp, u32, vp, vp]
+    L.srf_render_frame_paced.argtypes = [vp, vp, P(FrameArgs), vp, vp, vp, vp, vp, P(u32), vp]
+    L.srf_field_inference_counted.argtypes = [vp, vp, u32, vp, vp, i32, u32, vp]
+    L.srf_field_input_gradient_counted.argtypes = [vp, vp, u32, vp, vp]
+    L.srf_field_eval_counted.argtypes = [vp, P(Field), vp, u32, vp, vp, i32, u32, vp]
     L.srf_frame_accumulate.argtypes = [P(i32 * 2), vp, vp, u32, i32, vp]
     L.srf_frame_tonemap.argtypes = [P(i32 * 2), f32, P(f32 * 4), vp, i32, i32, i32, vp, vp]
     L.srf_debug_eval_elem.argtypes = [i32, u32, vp, vp, vp, vp]

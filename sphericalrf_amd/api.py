@@ -339,12 +339,14 @@ class OccupancySampler:
 
     def render_frame(self, marcher, inference, resolution, focal_length, principal_point, camera_matrix, frame_buffer, spp=0,
                      render_mode=K.RENDER_SHADE, density_activation=K.ACT_EXPONENTIAL, rgb_activation=K.ACT_LOGISTIC, depth_scale=1.0,
-                     network_output_dtype=K.DTYPE_F16, padded_output_width=4, input_gradient=None):
+                     network_output_dtype=K.DTYPE_F16, padded_output_width=4, input_gradient=None, paced=False):
         """Testbed::render_frame up to shade (internal/testbed.cu:479-611).  `inference` is a Field (the stand-in network) or a callable
         (n_elements, coords_ptr, rgbsigma_ptr, dtype, padded_output_width, stream_ptr) -> int that enqueues the network on the stream.
         Normals mode needs `input_gradient` (testbed.cu:558-560): True with a Field (the stand-in's gradient), else a callable
         (n_elements, coords_ptr, stream_ptr) -> int that overwrites each record's position with the density's gradient.
-        An exception raised by a callable ends the frame and is raised again here.  Returns the number of rounds."""
+        An exception raised by a callable ends the frame and is raised again here.  Returns the number of rounds.
+        paced=True runs the loop paced by the device (srf_render_frame_paced): the callables then get the element count as a device
+        pointer followed by an upper limit, (n_elements_ptr, max_elements, coords_ptr, ...), and must not need it on the host."""
         a = K.FrameArgs()
         a.resolution, a.focal_length, a.principal_point = (K.i32 * 2)(*resolution), (K.f32 * 2)(*focal_length), (K.f32 * 2)(*principal_point)
         a.camera_matrix = (K.f32 * 12)(*[float(v) for v in camera_matrix])
@@ -366,22 +368,36 @@ class OccupancySampler:
         if isinstance(inference, Field):
             f = inference.as_c()
             ctx = K.FieldInferenceCtx(self._h, C.pointer(f))
-            fn, user = C.cast(self._L.srf_field_inference, C.c_void_p), C.cast(C.pointer(ctx), C.c_void_p)
+            fn = C.cast(self._L.srf_field_inference_counted if paced else self._L.srf_field_inference, C.c_void_p)
+            user = C.cast(C.pointer(ctx), C.c_void_p)
             keep += [f, ctx]
             if input_gradient is True:
-                a.input_gradient, a.input_gradient_user = C.cast(self._L.srf_field_input_gradient, C.c_void_p), user
+                gfn, guser = C.cast(self._L.srf_field_input_gradient_counted if paced else self._L.srf_field_input_gradient, C.c_void_p), user
                 input_gradient = None
+            else:
+                gfn, guser = None, None
         else:
-            cb = K.INFERENCE_FN(lambda user, n_el, coords, out, dtype, width, stream: guarded(inference, n_el, coords, out, dtype, width, stream))
-            fn, user = C.cast(cb, C.c_void_p), None
+            if paced:
+                cb = K.INFERENCE_COUNTED_FN(lambda user, n_dev, n_max, coords, out, dtype, width, stream: guarded(inference, n_dev, n_max, coords, out, dtype, width, stream))
+            else:
+                cb = K.INFERENCE_FN(lambda user, n_el, coords, out, dtype, width, stream: guarded(inference, n_el, coords, out, dtype, width, stream))
+            fn, user, gfn, guser = C.cast(cb, C.c_void_p), None, None, None
             keep.append(cb)
         if input_gradient is True:
             raise ValueError("input_gradient=True needs a Field as the inference")
         if input_gradient is not None:
-            gcb = K.INPUT_GRADIENT_FN(lambda user, n_el, coords, stream: guarded(input_gradient, n_el, coords, stream))
-            a.input_gradient = C.cast(gcb, C.c_void_p)
+            if paced:
+                gcb = K.INPUT_GRADIENT_COUNTED_FN(lambda user, n_dev, n_max, coords, stream: guarded(input_gradient, n_dev, n_max, coords, stream))
+            else:
+                gcb = K.INPUT_GRADIENT_FN(lambda user, n_el, coords, stream: guarded(input_gradient, n_el, coords, stream))
+            gfn = C.cast(gcb, C.c_void_p)
             keep.append(gcb)
-        rc = self._L.srf_render_frame(self._h, marcher._h, C.byref(a), fn, user, _dev(frame_buffer, torch.float32, 4 * n, "frame_buffer"), C.byref(iters), _stream())
+        fb = _dev(frame_buffer, torch.float32, 4 * n, "frame_buffer")
+        if paced:
+            rc = self._L.srf_render_frame_paced(self._h, marcher._h, C.byref(a), fn, user, gfn, guser, fb, C.byref(iters), _stream())
+        else:
+            a.input_gradient, a.input_gradient_user = gfn, guser
+            rc = self._L.srf_render_frame(self._h, marcher._h, C.byref(a), fn, user, fb, C.byref(iters), _stream())
         del keep
         if raised:
             raise raised[0]

@@ -988,6 +988,7 @@ struct AdvanceMarch {
 // whatever its size.
 struct CoordsMarch {
 	MarchGrid G; uint32_t n_rays, n_steps; srf_ray_payload* payloads; float* coords;
+	const uint32_t* round = nullptr;      // device words {rays, steps} that replace n_rays and n_steps when the kernel starts (the frame loop paced by the device)
 	struct Lane { MarchLane m; uint32_t i, j; Vec3 wdir; };
 	struct Hit {
 		float* c; uint32_t* j; uint32_t n_steps; Vec3 wdir;

@@ -31,9 +31,12 @@ __global__ void __launch_bounds__(128) k_loss_backward(LossConst K, const uint32
 	                                                        mean_density_ptr ? *mean_density_ptr : 0.f, fwd[i], n_fwd[i], cbase_arr[i], reg_buffer);
 }
 
+// round: the frame loop's words on the device, in place of the three numbers of A that change from round to round (or NULL)
 template <bool HALF_IN>
 __global__ void __launch_bounds__(128) k_volume_rendering(Params P, srf_render_args A, float thr, srf_ray_payload* __restrict__ payloads,
-                                                          float* __restrict__ rgba, const float* __restrict__ coords, const void* __restrict__ net) {
+                                                          float* __restrict__ rgba, const float* __restrict__ coords, const void* __restrict__ net,
+                                                          const RoundWords* __restrict__ round) {
+	if (round) { A.n_rays = round->n_alive; A.n_steps = round->n_steps; A.i_steps_offset = round->offset; }
 	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
 	if (i < A.n_rays) volume_rendering_body<HALF_IN>(i, P, A, thr, payloads, rgba, coords, net);
 }
@@ -498,10 +501,18 @@ __device__ __forceinline__ uint32_t compact_class(uint32_t i, uint32_t n, const 
 }
 
 // counts[b] = {alive, finished} of block b; block 0 also notes the counters' values on entry, which are where this call's output starts
+// the number of rays a paced compaction looks at: those alive after the last round, none once the loop has run out of iterations
+__device__ __forceinline__ uint32_t paced_n(const RoundWords* __restrict__ in) { return in->next_offset < FRAME_MARCH_ITER ? in->n_alive : 0u; }
+
 __global__ void __launch_bounds__(COMPACT_BLOCK) k_compact_count(uint32_t n, const srf_ray_payload* __restrict__ payloads, const float* __restrict__ rgba,
                                                                  U2* __restrict__ counts, const uint32_t* __restrict__ n_alive_counter,
-                                                                 const uint32_t* __restrict__ n_final_counter, uint32_t* __restrict__ initial, bool alive_from_zero) {
+                                                                 const uint32_t* __restrict__ n_final_counter, uint32_t* __restrict__ initial, bool alive_from_zero,
+                                                                 const RoundWords* __restrict__ paced_in) {
 	__shared__ uint32_t part[2][COMPACT_BLOCK / 64];
+	if (paced_in) {
+		n = paced_n(paced_in);
+		if (blockIdx.x * COMPACT_BLOCK >= n && blockIdx.x != 0) return;      // (uniform over the block)
+	}
 	const uint32_t i = blockIdx.x * COMPACT_BLOCK + threadIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
 	const uint32_t c = compact_class(i, n, payloads, rgba);
 	const uint32_t na = (uint32_t)__popcll(__ballot(c == 1u)), nf = (uint32_t)__popcll(__ballot(c == 2u));
@@ -512,7 +523,7 @@ __global__ void __launch_bounds__(COMPACT_BLOCK) k_compact_count(uint32_t n, con
 		for (uint32_t k = 0; k < COMPACT_BLOCK / 64; ++k) { a += part[0][k]; f += part[1][k]; }
 		U2 v; v.x = a; v.y = f;
 		counts[blockIdx.x] = v;
-		if (blockIdx.x == 0) { initial[0] = alive_from_zero ? 0u : *n_alive_counter; initial[1] = *n_final_counter; }
+		if (blockIdx.x == 0) { initial[0] = alive_from_zero || paced_in ? 0u : *n_alive_counter; initial[1] = *n_final_counter; }
 	}
 }
 
@@ -521,10 +532,17 @@ __global__ void __launch_bounds__(COMPACT_BLOCK) k_compact_move(uint32_t n, cons
                                                                 srf_ray_payload* __restrict__ fin_p, float* __restrict__ fin_c,
                                                                 const U2* __restrict__ counts, const uint32_t* __restrict__ initial,
                                                                 uint32_t* __restrict__ n_alive_counter, uint32_t* __restrict__ n_final_counter,
-                                                                unsigned long long* __restrict__ host_word, uint32_t stamp) {
+                                                                unsigned long long* __restrict__ host_word, uint32_t stamp,
+                                                                const RoundWords* __restrict__ paced_in, RoundWords* __restrict__ paced_out, uint32_t n_pixels) {
 	__shared__ uint32_t part[2][COMPACT_BLOCK / 64];
 	__shared__ uint32_t before[2][COMPACT_BLOCK / 64];
 	__shared__ uint32_t block_base[2];
+	uint32_t last_block = gridDim.x - 1;
+	if (paced_in) {
+		n = paced_n(paced_in);
+		last_block = n ? (n - 1u) / COMPACT_BLOCK : 0u;
+		if (blockIdx.x > last_block) return;      // (uniform over the block)
+	}
 	const uint32_t i = blockIdx.x * COMPACT_BLOCK + threadIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
 	// what the blocks before this one hold
 	uint32_t a = 0, f = 0;
@@ -541,8 +559,23 @@ __global__ void __launch_bounds__(COMPACT_BLOCK) k_compact_move(uint32_t n, cons
 		// the wavefronts' offsets inside the block, in place of their counts
 		uint32_t run = 0;
 		for (uint32_t k = 0; k < COMPACT_BLOCK / 64; ++k) { const uint32_t v = part[threadIdx.x][k]; part[threadIdx.x][k] = run; run += v; }
-		if (blockIdx.x == gridDim.x - 1) {
-			*(threadIdx.x == 0 ? n_alive_counter : n_final_counter) = sum + run;
+		if (blockIdx.x == last_block) {
+			if (!paced_in) *(threadIdx.x == 0 ? n_alive_counter : n_final_counter) = sum + run;
+			else if (threadIdx.x == 1) *n_final_counter = sum + run;
+			else {
+				// the round's words (Testbed::render_frame's host arithmetic, testbed.cu:526-547, :596)
+				RoundWords w;
+				w.n_alive = sum + run;
+				uint32_t steps = w.n_alive ? n_pixels / w.n_alive : 0u;
+				steps = steps < FRAME_MIN_STEPS ? FRAME_MIN_STEPS : (steps > FRAME_MAX_STEPS ? FRAME_MAX_STEPS : steps);
+				w.n_steps = w.n_alive ? steps : 0u;
+				w.offset = paced_in->next_offset;
+				w.n_elements = w.n_alive * w.n_steps;
+				w.next_offset = w.offset + w.n_steps;
+				w.rounds = paced_in->rounds + (w.n_alive ? 1u : 0u);
+				w.pad[0] = w.pad[1] = 0u;
+				*paced_out = w;
+			}
 			// for a host that waits for the number of live rays: the count with the call's stamp above it, in one store to host memory
 			if (threadIdx.x == 0 && host_word) __hip_atomic_store(host_word, ((unsigned long long)stamp << 32) | (sum + run), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 		}
@@ -561,7 +594,8 @@ __global__ void __launch_bounds__(COMPACT_BLOCK) k_compact_move(uint32_t n, cons
 }
 
 __global__ void __launch_bounds__(256) k_shade(uint32_t n, const float* __restrict__ rgba, const srf_ray_payload* __restrict__ payloads,
-                                               float* __restrict__ frame, int render_mode, int train_in_linear) {
+                                               float* __restrict__ frame, int render_mode, int train_in_linear, const uint32_t* __restrict__ n_dev) {
+	if (n_dev) n = *n_dev;
 	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
 	if (i < n) shade_body(i, rgba, payloads, frame, render_mode, train_in_linear);
 }
@@ -691,10 +725,47 @@ int compact_rays(srf_marcher* m, uint32_t n, const srf_ray_payload* src_payloads
 	uint32_t* initial = (uint32_t*)m->compact_ws.ptr;
 	U2* counts = (U2*)((char*)m->compact_ws.ptr + 256);
 	hipLaunchKernelGGL(k_compact_count, dim3(blocks), dim3(COMPACT_BLOCK), 0, st, n, src_payloads, src_rgba, counts,
-	                   (const uint32_t*)n_alive_counter, (const uint32_t*)n_final_counter, initial, alive_from_zero);
+	                   (const uint32_t*)n_alive_counter, (const uint32_t*)n_final_counter, initial, alive_from_zero, (const RoundWords*)nullptr);
 	SRF_LAUNCH_CHECK();
 	hipLaunchKernelGGL(k_compact_move, dim3(blocks), dim3(COMPACT_BLOCK), 0, st, n, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba,
-	                   (const U2*)counts, (const uint32_t*)initial, n_alive_counter, n_final_counter, host_word, stamp);
+	                   (const U2*)counts, (const uint32_t*)initial, n_alive_counter, n_final_counter, host_word, stamp, (const RoundWords*)nullptr, (RoundWords*)nullptr, 0u);
+	SRF_LAUNCH_CHECK();
+	return SRF_OK;
+}
+
+int compact_rays_paced(srf_marcher* m, uint32_t bound, uint32_t n_pixels, const RoundWords* in, RoundWords* out, const srf_ray_payload* src_payloads, const float* src_rgba,
+                       srf_ray_payload* dst_payloads, float* dst_rgba, srf_ray_payload* final_payloads, float* final_rgba, uint32_t* n_final_counter,
+                       hipStream_t st, unsigned long long* host_word, uint32_t stamp) {
+	const uint32_t blocks = div_up(bound ? bound : 1u, COMPACT_BLOCK);      // block 0 always runs: it writes the round's words
+	int rc = m->compact_ws.reserve(256 + (size_t)div_up(n_pixels, COMPACT_BLOCK) * sizeof(U2));
+	if (rc != SRF_OK) return rc;
+	uint32_t* initial = (uint32_t*)m->compact_ws.ptr;
+	U2* counts = (U2*)((char*)m->compact_ws.ptr + 256);
+	hipLaunchKernelGGL(k_compact_count, dim3(blocks), dim3(COMPACT_BLOCK), 0, st, 0u, src_payloads, src_rgba, counts,
+	                   (const uint32_t*)nullptr, (const uint32_t*)n_final_counter, initial, true, in);
+	SRF_LAUNCH_CHECK();
+	hipLaunchKernelGGL(k_compact_move, dim3(blocks), dim3(COMPACT_BLOCK), 0, st, 0u, src_payloads, src_rgba, dst_payloads, dst_rgba, final_payloads, final_rgba,
+	                   (const U2*)counts, (const uint32_t*)initial, (uint32_t*)nullptr, n_final_counter, host_word, stamp, in, out, n_pixels);
+	SRF_LAUNCH_CHECK();
+	return SRF_OK;
+}
+
+int volume_rendering_paced(srf_marcher* m, const srf_sampler* s, const srf_render_args* a, uint32_t bound, const RoundWords* round,
+                           srf_ray_payload* payloads, float* rgba, const float* coords, const void* rgbsigma, hipStream_t st) {
+	if (bound == 0) return SRF_OK;
+	const dim3 grid(div_up(bound, 128)), block(128);
+	if (a->network_output_dtype == SRF_DTYPE_F16)
+		hipLaunchKernelGGL(k_volume_rendering<true>, grid, block, 0, st, s->P, *a, m->cfg.transmittance_threshold, payloads, rgba, coords, rgbsigma, round);
+	else
+		hipLaunchKernelGGL(k_volume_rendering<false>, grid, block, 0, st, s->P, *a, m->cfg.transmittance_threshold, payloads, rgba, coords, rgbsigma, round);
+	SRF_LAUNCH_CHECK();
+	return SRF_OK;
+}
+
+int shade_counted(uint32_t bound, const uint32_t* n_rays, const float* rgba, const srf_ray_payload* payloads, float* frame_buffer,
+                  int32_t render_mode, int32_t train_in_linear_colors, hipStream_t st) {
+	if (bound == 0) return SRF_OK;
+	hipLaunchKernelGGL(k_shade, dim3(div_up(bound, 256)), dim3(256), 0, st, bound, rgba, payloads, frame_buffer, render_mode, train_in_linear_colors, n_rays);
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }
@@ -967,9 +1038,9 @@ int srf_marcher_volume_rendering(srf_marcher_t* m, const srf_sampler_t* s, const
 	SRF_REQUIRE((a->network_output_dtype | 1) == 1, "srf_marcher_volume_rendering: unknown dtype");
 	const dim3 grid(div_up(a->n_rays, 128)), block(128);
 	if (a->network_output_dtype == SRF_DTYPE_F16)
-		hipLaunchKernelGGL(k_volume_rendering<true>, grid, block, 0, (hipStream_t)stream, s->P, *a, m->cfg.transmittance_threshold, payloads, rgba, coords, rgbsigma);
+		hipLaunchKernelGGL(k_volume_rendering<true>, grid, block, 0, (hipStream_t)stream, s->P, *a, m->cfg.transmittance_threshold, payloads, rgba, coords, rgbsigma, (const RoundWords*)nullptr);
 	else
-		hipLaunchKernelGGL(k_volume_rendering<false>, grid, block, 0, (hipStream_t)stream, s->P, *a, m->cfg.transmittance_threshold, payloads, rgba, coords, rgbsigma);
+		hipLaunchKernelGGL(k_volume_rendering<false>, grid, block, 0, (hipStream_t)stream, s->P, *a, m->cfg.transmittance_threshold, payloads, rgba, coords, rgbsigma, (const RoundWords*)nullptr);
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }
@@ -984,7 +1055,7 @@ int srf_shade(uint32_t n_rays, const float* rgba, const srf_ray_payload* payload
               int32_t render_mode, int32_t train_in_linear_colors, void* stream) {
 	if (n_rays == 0) return SRF_OK;
 	SRF_REQUIRE(rgba && payloads && frame_buffer, "srf_shade: NULL buffer");
-	hipLaunchKernelGGL(k_shade, dim3(div_up(n_rays, 256)), dim3(256), 0, (hipStream_t)stream, n_rays, rgba, payloads, frame_buffer, render_mode, train_in_linear_colors);
+	hipLaunchKernelGGL(k_shade, dim3(div_up(n_rays, 256)), dim3(256), 0, (hipStream_t)stream, n_rays, rgba, payloads, frame_buffer, render_mode, train_in_linear_colors, (const uint32_t*)nullptr);
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }

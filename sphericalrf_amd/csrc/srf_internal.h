@@ -99,6 +99,29 @@ uint32_t* waves_error_word(void* scratch);
 int launch_waves(const srf_loss_args* a, const LossConst& K, void* scratch, uint32_t* host_error, uint32_t spin_limit, const float* rays_rgba, const uint32_t* n_rays_counter,
                  uint32_t* ray_coord_indices, const float* dt, const float* coords, float* compacted_coords, uint32_t* n_compacted_coords_counter,
                  const void* network_output, void* dloss_doutput, float* loss_output, const float* density_grid_mean, float* rgb_ray_out, hipStream_t st);
+// ---- the frame loop paced by the device (srf_render_frame_paced) ----
+// What a round of the loop needs to know, kept on the device: the compaction of round r reads the words of round r - 1 and writes
+// those of round r (two sets that take turns), every other kernel of round r reads the latter.
+struct RoundWords {
+	uint32_t n_alive;       // rays alive after this round's compaction (0: the frame is finished, every later kernel returns at once)
+	uint32_t n_steps;       // clamp(n_pixels / n_alive, 1, 8), testbed.cu:544-547
+	uint32_t offset;        // i_steps_offset of this round's volume_rendering
+	uint32_t n_elements;    // n_alive * n_steps: what the network evaluates
+	uint32_t next_offset;   // offset + n_steps; the loop ends once it reaches MARCH_ITER (testbed.cu:526)
+	uint32_t rounds;        // rounds with live rays so far
+	uint32_t pad[2];
+};
+constexpr uint32_t FRAME_MARCH_ITER = 10000, FRAME_MIN_STEPS = 1, FRAME_MAX_STEPS = 8;      // testbed.h: MARCH_ITER, MIN/MAX_STEPS_INBETWEEN_COMPACTION
+// bound: an upper limit of the rays the call has to look at, known to the host; the kernels take the true numbers from the words
+int compact_rays_paced(srf_marcher* m, uint32_t bound, uint32_t n_pixels, const RoundWords* in, RoundWords* out, const srf_ray_payload* src_payloads, const float* src_rgba,
+                       srf_ray_payload* dst_payloads, float* dst_rgba, srf_ray_payload* final_payloads, float* final_rgba, uint32_t* n_final_counter,
+                       hipStream_t stream, unsigned long long* host_word, uint32_t stamp);
+int generate_coords_paced(srf_sampler* s, uint32_t bound, const RoundWords* round, srf_ray_payload* payloads, float* coords, hipStream_t stream);
+int volume_rendering_paced(srf_marcher* m, const srf_sampler* s, const srf_render_args* a, uint32_t bound, const RoundWords* round,
+                           srf_ray_payload* payloads, float* rgba, const float* coords, const void* rgbsigma, hipStream_t stream);
+int shade_counted(uint32_t bound, const uint32_t* n_rays, const float* rgba, const srf_ray_payload* payloads, float* frame_buffer,
+                  int32_t render_mode, int32_t train_in_linear_colors, hipStream_t stream);
+
 // srf_compact_rays with two more choices: alive_from_zero numbers the live rays from 0 whatever *n_alive_counter holds; host_word
 // (device address of a word of host memory, or NULL) receives stamp << 32 | the live-ray counter's new value when the call is done
 int compact_rays(srf_marcher* m, uint32_t n, const srf_ray_payload* src_payloads, const float* src_rgba,

@@ -303,9 +303,14 @@ __device__ inline bool march_wide_round(const MarchGrid& G, MarchLane& L, uint32
 	return m == 0ull;
 }
 
+// numbers that a march takes from device memory when its kernels start, where the host only knows an upper limit of them
+template <class March> __device__ __forceinline__ void march_resolve(March&) {}
+__device__ __forceinline__ void march_resolve(CoordsMarch& M) { if (M.round) { M.n_rays = M.round[0]; M.n_steps = M.round[1]; } }
+
 // the parked rays, one a wavefront: lane 0 carries the ray's state and runs its probes and steps, all lanes its wide rounds
 template <class March>
 __global__ void __launch_bounds__(64) k_march_wide(March M, MarchPark park) {
+	march_resolve(M);
 	const uint32_t lane = threadIdx.x;
 	const uint32_t filled = *park.count;
 	const uint32_t n = filled < park.capacity ? filled : park.capacity;
@@ -332,6 +337,7 @@ __device__ unsigned long long g_march_timing[16];
 #endif
 template <class March>
 __global__ void __launch_bounds__(64) k_march_lanes(March M, MarchPark park) {
+	march_resolve(M);
 	const uint32_t q = blockIdx.x * 64u + threadIdx.x;
 	typename March::Lane L;
 	L.m.phase = LANE_IDLE;
@@ -426,7 +432,9 @@ __global__ void __launch_bounds__(256) k_ray_sphere_bounds(uint32_t n_rays, cons
 }
 
 template <bool HALF>
-__global__ void __launch_bounds__(256) k_field_eval(Params P, uint32_t n, const float* __restrict__ coords, FieldArgs F, void* __restrict__ out, uint32_t width) {
+__global__ void __launch_bounds__(256) k_field_eval(Params P, uint32_t n, const float* __restrict__ coords, FieldArgs F, void* __restrict__ out, uint32_t width,
+                                                    const uint32_t* __restrict__ n_dev) {
+	if (n_dev) n = *n_dev;
 	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
 	if (i < n) field_eval_body<HALF>(i, P, coords, F, out, width);
 }
@@ -635,6 +643,20 @@ int srf_sampler_generate_rays_from_camera_matrix(srf_sampler_t* s, const int32_t
 	return launch_march(M, s, st);
 }
 
+} // extern "C"
+
+namespace srf {
+int generate_coords_paced(srf_sampler* s, uint32_t bound, const RoundWords* round, srf_ray_payload* payloads, float* coords, hipStream_t stream) {
+	if (bound == 0) return SRF_OK;
+	CoordsMarch M;
+	M.G = sampler_march_grid(s); M.n_rays = bound; M.n_steps = FRAME_MAX_STEPS; M.payloads = payloads; M.coords = coords;
+	M.round = &round->n_alive;      // {n_alive, n_steps}
+	return launch_march(M, s, stream);
+}
+} // namespace srf
+
+extern "C" {
+
 int srf_sampler_generate_coords_from_rays(srf_sampler_t* s, uint32_t n_rays, uint32_t n_steps,
                                           srf_ray_payload* payloads, float* coords, void* stream) {
 	SRF_REQUIRE(s, "srf_sampler_generate_coords_from_rays: NULL sampler");
@@ -647,6 +669,11 @@ int srf_sampler_generate_coords_from_rays(srf_sampler_t* s, uint32_t n_rays, uin
 
 int srf_field_eval(const srf_sampler_t* s, const srf_field* field, uint32_t n_coords, const float* coords,
                    void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream) {
+	return srf_field_eval_counted(s, field, nullptr, n_coords, coords, rgbsigma, dtype, padded_output_width, stream);
+}
+
+int srf_field_eval_counted(const srf_sampler_t* s, const srf_field* field, const uint32_t* n_coords_dev, uint32_t n_coords, const float* coords,
+                           void* rgbsigma, int32_t dtype, uint32_t padded_output_width, void* stream) {
 	SRF_REQUIRE(s && field && field->table, "srf_field_eval: NULL argument");
 	SRF_REQUIRE(field->table_size && !(field->table_size & (field->table_size - 1)), "srf_field_eval: table_size must be a power of two");
 	SRF_REQUIRE(padded_output_width >= 4, "srf_field_eval: padded_output_width must be >= 4");
@@ -656,9 +683,9 @@ int srf_field_eval(const srf_sampler_t* s, const srf_field* field, uint32_t n_co
 	SRF_REQUIRE(coords && rgbsigma, "srf_field_eval: NULL buffer");
 	FieldArgs F; F.table = field->table; F.mask = field->table_size - 1; F.seed = field->seed;
 	if (dtype == SRF_DTYPE_F16)
-		hipLaunchKernelGGL(k_field_eval<true>, dim3(div_up(n_coords, 256)), dim3(256), 0, (hipStream_t)stream, s->P, n_coords, coords, F, rgbsigma, padded_output_width);
+		hipLaunchKernelGGL(k_field_eval<true>, dim3(div_up(n_coords, 256)), dim3(256), 0, (hipStream_t)stream, s->P, n_coords, coords, F, rgbsigma, padded_output_width, n_coords_dev);
 	else
-		hipLaunchKernelGGL(k_field_eval<false>, dim3(div_up(n_coords, 256)), dim3(256), 0, (hipStream_t)stream, s->P, n_coords, coords, F, rgbsigma, padded_output_width);
+		hipLaunchKernelGGL(k_field_eval<false>, dim3(div_up(n_coords, 256)), dim3(256), 0, (hipStream_t)stream, s->P, n_coords, coords, F, rgbsigma, padded_output_width, n_coords_dev);
 	SRF_LAUNCH_CHECK();
 	return SRF_OK;
 }

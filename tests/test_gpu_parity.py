@@ -781,10 +781,12 @@ def test_render_loop_and_fused_frame(gpu, orc, config_id, scale):
     assert np.array_equal(fb.cpu().numpy(), want_frame)
 
 
+@pytest.mark.parametrize("paced", [False, True])
 @pytest.mark.parametrize("config_id,scale,inference", [(1, 0.5, "field"), (3, 0.125, "field"), (1, 0.25, "callback")])
-def test_library_side_frame_loop(gpu, orc, config_id, scale, inference):
+def test_library_side_frame_loop(gpu, orc, config_id, scale, inference, paced):
     """srf_render_frame (internal/testbed.cu:479-611) with the stand-in field as the network, handed over as the library's own
-    inference function or as a caller's callback: frame and number of rounds against the oracle's loop"""
+    inference function or as a caller's callback: frame and number of rounds against the oracle's loop; with the host pacing the
+    rounds as the reference does, and with the device pacing them (srf_render_frame_paced)"""
     torch = gpu
     from sphericalrf_amd import api, scene, _capi
     w, p, grid, bf, mean = helpers.build_scene(orc, config_id, scale)
@@ -802,19 +804,27 @@ def test_library_side_frame_loop(gpu, orc, config_id, scale, inference):
         def net(n_elements, coords, out, dtype, width, stream):      # a caller's network: raw device pointers in, work enqueued on the stream
             calls.append(n_elements)
             return _capi.load().srf_field_eval(s._h, fc, n_elements, coords, out, dtype, width, stream)
+
+        def net_counted(n_elements_dev, max_elements, coords, out, dtype, width, stream):      # the count stays on the device
+            calls.append(max_elements)
+            return _capi.load().srf_field_eval_counted(s._h, fc, n_elements_dev, max_elements, coords, out, dtype, width, stream)
+        if paced:
+            net = net_counted
     else:
         net = field
     frame = torch.ones((res[1], res[0], 4), device="cuda")
     for rep in range(2):        # the second frame reuses the marcher's buffers
         got_iters = s.render_frame(m, net, res, f, (0.5, 0.5), cam, frame, density_activation=api.ACT_NONE, rgb_activation=api.ACT_NONE,
-                                   network_output_dtype=api.DTYPE_F32)
+                                   network_output_dtype=api.DTYPE_F32, paced=paced)
         assert got_iters == iters and np.array_equal(frame.cpu().numpy(), want_frame)
-    assert inference != "callback" or len(calls) == 2 * iters
+    if inference == "callback":        # the paced loop may have launched a few rounds past the end (they return at once)
+        assert len(calls) == 2 * iters if not paced else 2 * iters <= len(calls) <= 2 * (iters + 8) and max(calls) <= res[0] * res[1]
     assert (want_frame[..., 3] > 0).mean() > 0.05
 
 
+@pytest.mark.parametrize("paced", [False, True])
 @pytest.mark.parametrize("mode", ["AO", "NORMALS", "DEPTH", "DISTANCE", "COST"])
-def test_library_side_frame_loop_in_every_render_mode(gpu, orc, mode):
+def test_library_side_frame_loop_in_every_render_mode(gpu, orc, mode, paced):
     """srf_render_frame in the other render modes (internal/testbed.cu:558-560 and :603-611): Normals mode overwrites a round's
     coordinates with the network's input gradient (here the stand-in's) before they are composited"""
     torch = gpu
@@ -833,13 +843,13 @@ def test_library_side_frame_loop_in_every_render_mode(gpu, orc, mode):
     field = api.Field(torch.from_numpy(table).cuda(), 77)
     frame = torch.ones((res[1], res[0], 4), device="cuda")
     got_iters = s.render_frame(m, field, res, f, (0.5, 0.5), cam, frame, render_mode=render_mode, density_activation=api.ACT_NONE, rgb_activation=api.ACT_NONE,
-                               network_output_dtype=api.DTYPE_F32, input_gradient=True if mode == "NORMALS" else None)
+                               network_output_dtype=api.DTYPE_F32, input_gradient=True if mode == "NORMALS" else None, paced=paced)
     assert got_iters == iters and np.array_equal(frame.cpu().numpy(), want_frame)
     if mode == "NORMALS":
         # without the gradient step the positions themselves would be composited: a different frame, so the mode is refused
         with pytest.raises(api.SrfError) as e:
             s.render_frame(m, field, res, f, (0.5, 0.5), cam, frame, render_mode=render_mode, density_activation=api.ACT_NONE, rgb_activation=api.ACT_NONE,
-                           network_output_dtype=api.DTYPE_F32)
+                           network_output_dtype=api.DTYPE_F32, paced=paced)
         assert e.value.code == api.ERR_UNSUPPORTED
 
 
