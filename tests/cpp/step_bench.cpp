@@ -1,9 +1,13 @@
 // Torch-free driver of one training step (march + compositing forward/backward) through include/srf_hip.hpp,
 // for timing and for profiler runs (a process that holds nothing but this library's kernels and a few fill kernels).
 //
-//   step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite|render] [--verify] [--copy-check]
+//   step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite|render|grid] [--verify] [--copy-check]
+//              [--cell-order] [--steady]
 //
 // --only render times whole frames of the workload file's cameras through srf_render_frame_fused instead (any workload).
+// --only grid times the occupancy-grid maintenance of the workload's grid (Testbed::train's calls, internal/testbed.cu:343-372):
+// sample_positions_from_grid, update_grid with one table density per point, update_grid_bitfield; one uniform point per cell as
+// in the reference's first 256 steps, or with --steady a quarter of the cells each way; --cell-order draws the points in cell order.
 //
 // The workload file (written by sphericalrf_amd.scene.write_workload_file) holds the sampler configuration, the
 // cameras, the occupancy bitfield and a table of (r, g, b, sigma) rows; per-sample network output and per-ray targets
@@ -49,6 +53,12 @@ __global__ void k_fill_network_output(const float* __restrict__ table, uint32_t 
 	const float4 row = ((const float4*)table)[mix32(s ^ seed) & table_mask];
 	__half* o = out + 4 * (size_t)s;
 	o[0] = __float2half(row.x); o[1] = __float2half(row.y); o[2] = __float2half(row.z); o[3] = __float2half(row.w);
+}
+
+// density of grid point i: the sigma column of row hash(i) of the table, as a half
+__global__ void k_fill_point_density(const float* __restrict__ table, uint32_t table_mask, uint32_t seed, uint32_t n, __half* __restrict__ out) {
+	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+	if (i < n) out[i] = __float2half(table[4 * (size_t)(mix32(i ^ seed) & table_mask) + 3]);
 }
 
 // target colour of ray i: uniform in [0, 1), alpha 1
@@ -104,9 +114,9 @@ struct Timer {
 };
 
 int main(int argc, char** argv) {
-	if (argc < 2) { std::fprintf(stderr, "usage: step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite|render] [--verify] [--copy-check]\n"); return 2; }
+	if (argc < 2) { std::fprintf(stderr, "usage: step_bench <workload file> [--steps K] [--warmup W] [--rays N] [--cap C] [--only march|composite|render|grid] [--verify] [--copy-check] [--cell-order] [--steady]\n"); return 2; }
 	uint32_t steps = 10, warmup = 2, n_rays = 1u << 20, cap = 1u << 24;
-	bool verify = false, copy_check = false;
+	bool verify = false, copy_check = false, cell_order = false, steady = false;
 	std::string only;
 	for (int i = 2; i < argc; ++i) {
 		const std::string a = argv[i];
@@ -118,6 +128,8 @@ int main(int argc, char** argv) {
 		else if (a == "--only") only = next();
 		else if (a == "--verify") verify = true;
 		else if (a == "--copy-check") copy_check = true;
+		else if (a == "--cell-order") cell_order = true;
+		else if (a == "--steady") steady = true;
 		else { std::fprintf(stderr, "unknown option %s\n", a.c_str()); return 2; }
 	}
 	const Workload w = load_workload(argv[1]);
@@ -148,6 +160,49 @@ int main(int argc, char** argv) {
 		mc.train_in_linear_color = 1;
 		mc.transmittance_threshold = 1e-4f;
 		srf::RayMarcher marcher(mc);
+
+		if (only == "grid") {
+			sampler.set_grid_sample_order(cell_order);
+			srf_pcg32 grid_rng{0x853c49e6748fea9bULL, 0xda3e39cb94b95bdbULL};
+			const float pp[2] = {0.5f, 0.5f};
+			sampler.init(1, w.res, w.focal, pp, nullptr, grid_rng, st);       // a grid without a camera mask starts from zero (occupancy_sampler.cu:946-978)
+			const uint32_t n_total = info.n_total_elements;
+			const uint32_t n_uni = steady ? n_total / 4 : n_total, n_non = steady ? n_total / 4 : 0u, n_points = n_uni + n_non;
+			float* pos = dev_alloc<float>((size_t)n_points * 3);
+			uint32_t* idx = dev_alloc<uint32_t>(n_points);
+			__half* dens = dev_alloc<__half>(n_points);
+			float* d_table = dev_alloc<float>(w.table.size());
+			HIP_OK(hipMemcpy(d_table, w.table.data(), w.table.size() * 4, hipMemcpyHostToDevice));
+			hipLaunchKernelGGL(k_fill_point_density, dim3((n_points + 255) / 256), dim3(256), 0, st, d_table, (uint32_t)(w.table.size() / 4 - 1), 49u, n_points, dens);
+			HIP_OK(hipStreamSynchronize(st));
+			Timer tm;
+			double ms[3] = {0, 0, 0};
+			for (uint32_t k = 0; k < warmup + steps; ++k) {
+				tm.start(st);
+				sampler.sample_positions_from_grid(n_uni, n_non, pos, idx, st);
+				const float t0 = tm.stop(st);
+				tm.start(st);
+				sampler.update_grid(n_points, 1, dens, SRF_DTYPE_F16, idx, SRF_ACT_NONE, st);
+				const float t1 = tm.stop(st);
+				tm.start(st);
+				sampler.update_grid_bitfield(st);
+				const float t2 = tm.stop(st);
+				if (k >= warmup) { ms[0] += t0; ms[1] += t1; ms[2] += t2; }
+			}
+			if (copy_check) {
+				const size_t n16 = (size_t)1 << 24;
+				uint4* src = dev_alloc<uint4>(n16);
+				uint4* dst = dev_alloc<uint4>(n16);
+				HIP_OK(hipMemset(src, 1, n16 * 16));
+				for (int k = 0; k < 3; ++k) hipLaunchKernelGGL(k_plain_copy, dim3(16384), dim3(256), 0, st, (const uint4*)src, dst, n16);
+				HIP_OK(hipStreamSynchronize(st));
+			}
+			std::printf("{\"cells\": %u, \"points\": %u, \"cell_order\": %s, \"steady_state\": %s, \"steps\": %u, \"sample_positions_ms\": %.4f, \"update_grid_ms\": %.4f, "
+			            "\"update_grid_bitfield_ms\": %.4f, \"update_grid_gbs\": %.1f, \"bitfield_gbs\": %.1f}\n", n_total, n_points, cell_order ? "true" : "false",
+			            steady ? "true" : "false", steps, ms[0] / steps, ms[1] / steps, ms[2] / steps, 12.0 * n_total / (ms[1] / steps * 1e-3) / 1e9,
+			            4.125 * n_total / (ms[2] / steps * 1e-3) / 1e9);
+			return 0;
+		}
 
 		if (only == "render") {
 			// frames of the workload's cameras in turn through the one-launch frame, the table standing in for the network
