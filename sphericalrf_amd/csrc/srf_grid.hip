@@ -203,6 +203,194 @@ __global__ void __launch_bounds__(256) k_splat_slabs(uint32_t n_elements, uint32
 	for (uint32_t j = threadIdx.x; j < SPLAT_SLAB_CELLS; j += 256u) if (first + j < n_total) grid_current_bits[first + j] = tile[j];
 }
 
+// The same without a sorting library: a partition by slab made for this job, in two levels of at most 256 and 64 parts so that
+// every level writes runs of some hundred bytes.  Which of a slab's samples comes first does not matter (the maximum does not depend
+// on the order), so nothing has to be stable.  k_part_count counts the samples of every slab (a histogram in LDS, flushed once
+// per workgroup); k_part_scan turns the counts into where each slab and each bucket of 64 slabs starts; k_part_pass<1> takes chunks
+// of 8192 samples, computes their (cell, thickness) pairs, reserves the chunk's share of every bucket's positions with one device
+// atomic per bucket, orders the pairs by bucket in LDS and writes them out run by run; k_part_pass<2> does the same by slab with the
+// chunks of one bucket at a time.  k_part_slabs then combines every slab in LDS as k_splat_slabs does, knows each slab's range from
+// the scan, and, where nothing else splats after it, applies the decay to the grid in the same pass (k_ema_grid's arithmetic).
+constexpr uint32_t PART_SLAB_BITS = 14;                    // 16384 cells: 64 KB of LDS per workgroup in k_part_slabs
+constexpr uint32_t PART_SLAB_CELLS = 1u << PART_SLAB_BITS;
+constexpr uint32_t PART_BUCKET_BITS = 6;                   // slabs per bucket
+constexpr uint32_t PART_BUCKET_SLABS = 1u << PART_BUCKET_BITS;
+constexpr uint32_t PART_MAX_BUCKETS = 256;
+constexpr uint32_t PART_MAX_SLABS = PART_MAX_BUCKETS * PART_BUCKET_SLABS;      // 16384 slabs = 2^28 cells
+constexpr uint32_t PART_THREADS = 1024;
+constexpr uint32_t PART_CHUNK = 8192, PART_PASS_THREADS = 512, PART_PER_THREAD = PART_CHUNK / PART_PASS_THREADS;
+
+__global__ void __launch_bounds__(PART_THREADS) k_part_count(uint32_t n, const uint32_t* __restrict__ indices, uint32_t n_total, uint32_t n_slabs, uint32_t* __restrict__ counts) {
+	extern __shared__ uint32_t part_h[];
+	for (uint32_t b = threadIdx.x; b < n_slabs; b += PART_THREADS) part_h[b] = 0u;
+	__syncthreads();
+	for (size_t i = (size_t)blockIdx.x * PART_THREADS + threadIdx.x; i < n; i += (size_t)gridDim.x * PART_THREADS) {
+		const uint32_t c = indices[i];
+		if (c < n_total) atomicAdd(&part_h[c >> PART_SLAB_BITS], 1u);
+	}
+	__syncthreads();
+	for (uint32_t b = threadIdx.x; b < n_slabs; b += PART_THREADS) { const uint32_t v = part_h[b]; if (v) atomicAdd(&counts[b], v); }
+}
+
+// What the scan leaves: starts[s] = samples in slabs before s (starts[n_slabs] = all), slab_cursor = a copy that pass 2 advances;
+// per bucket b: bucket_cursor[b] = starts[64 b] (advanced by pass 1), chunk_first[b] = chunks of 8192 in the buckets before b.
+struct PartTables { uint32_t* starts; uint32_t* slab_cursor; uint32_t* bucket_cursor; uint32_t* chunk_first; };
+__global__ void __launch_bounds__(PART_THREADS) k_part_scan(uint32_t n_slabs, uint32_t n_buckets, const uint32_t* __restrict__ counts, PartTables T) {
+	__shared__ uint32_t sums[PART_THREADS];
+	const uint32_t per = div_up(n_slabs, PART_THREADS);
+	const uint32_t lo = threadIdx.x * per, hi = lo + per < n_slabs ? lo + per : n_slabs;
+	uint32_t run = 0;
+	for (uint32_t b = lo; b < hi; ++b) run += counts[b];
+	sums[threadIdx.x] = run;
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		uint32_t acc = 0;
+		for (uint32_t k = 0; k < PART_THREADS; ++k) { const uint32_t v = sums[k]; sums[k] = acc; acc += v; }
+		T.starts[n_slabs] = acc;
+	}
+	__syncthreads();
+	run = sums[threadIdx.x];
+	for (uint32_t b = lo; b < hi; ++b) { T.starts[b] = run; T.slab_cursor[b] = run; run += counts[b]; }
+	__syncthreads();
+	// per bucket (starts were written by other threads of this workgroup: visible after the barrier)
+	uint32_t my_chunks = 0;
+	if (threadIdx.x < n_buckets) {
+		const uint32_t b = threadIdx.x;
+		const uint32_t s0 = b << PART_BUCKET_BITS, s1 = s0 + PART_BUCKET_SLABS < n_slabs ? s0 + PART_BUCKET_SLABS : n_slabs;
+		const uint32_t first = ((volatile uint32_t*)T.starts)[s0], size = ((volatile uint32_t*)T.starts)[s1] - first;
+		T.bucket_cursor[b] = first;
+		my_chunks = div_up(size, PART_CHUNK);
+	}
+	sums[threadIdx.x] = my_chunks;
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		uint32_t chunks = 0;
+		for (uint32_t b = 0; b < n_buckets; ++b) { T.chunk_first[b] = chunks; chunks += sums[b]; }
+		T.chunk_first[n_buckets] = chunks;
+	}
+}
+
+// One level of the partition.  LEVEL 1: input = the caller's arrays, part = bucket of the cell's slab, one chunk = 8192 consecutive
+// samples.  LEVEL 2: input = pass 1's pairs, part = slab within the bucket, chunks numbered bucket by bucket (chunk_first).
+template <int LEVEL, bool HALF>
+__global__ void __launch_bounds__(PART_PASS_THREADS) k_part_pass(uint32_t n, const uint32_t* __restrict__ indices, uint32_t width, const void* __restrict__ densities, int act,
+                                                                 float min_cone_stepsize, uint32_t n_total, uint32_t n_slabs, uint32_t n_buckets, PartTables T,
+                                                                 const U2* __restrict__ in_pairs, U2* __restrict__ out_pairs) {
+	__shared__ U2 stage[PART_CHUNK];
+	__shared__ uint32_t hist[PART_MAX_BUCKETS], lstart[PART_MAX_BUCKETS + 1], gbase[PART_MAX_BUCKETS], fill[PART_MAX_BUCKETS];
+	constexpr uint32_t NONE = 0xffffffffu;
+	const uint32_t n_parts = LEVEL == 1 ? n_buckets : PART_BUCKET_SLABS;
+	const uint32_t n_chunks = LEVEL == 1 ? div_up(n, PART_CHUNK) : ((volatile const uint32_t*)T.chunk_first)[n_buckets];
+	for (uint32_t w = blockIdx.x; w < n_chunks; w += gridDim.x) {
+		size_t first, last;
+		uint32_t bucket = 0;
+		if (LEVEL == 1) {
+			first = (size_t)w * PART_CHUNK;
+			last = first + PART_CHUNK < n ? first + PART_CHUNK : n;
+		} else {
+			uint32_t lo = 0, hi = n_buckets;      // the bucket whose chunks include w: the last b with chunk_first[b] <= w
+			while (hi - lo > 1u) { const uint32_t mid = (lo + hi) / 2u; if (T.chunk_first[mid] <= w) lo = mid; else hi = mid; }
+			bucket = lo;
+			const uint32_t s0 = bucket << PART_BUCKET_BITS, s1 = s0 + PART_BUCKET_SLABS < n_slabs ? s0 + PART_BUCKET_SLABS : n_slabs;
+			const size_t b_first = T.starts[s0], b_last = T.starts[s1];
+			first = b_first + (size_t)(w - T.chunk_first[bucket]) * PART_CHUNK;
+			last = first + PART_CHUNK < b_last ? first + PART_CHUNK : b_last;
+		}
+		if (threadIdx.x < PART_MAX_BUCKETS) { hist[threadIdx.x] = 0u; fill[threadIdx.x] = 0u; }
+		__syncthreads();
+		U2 e[PART_PER_THREAD];
+		uint32_t part[PART_PER_THREAD];
+		#pragma unroll
+		for (uint32_t k = 0; k < PART_PER_THREAD; ++k) {
+			const size_t i = first + (size_t)k * PART_PASS_THREADS + threadIdx.x;
+			part[k] = NONE;
+			if (i < last) {
+				if (LEVEL == 1) {
+					e[k].x = indices[i];
+					e[k].y = srf_f2u(act_density(net_load<HALF>(densities, i * width), act) * min_cone_stepsize);
+					if (e[k].x < n_total) part[k] = e[k].x >> (PART_SLAB_BITS + PART_BUCKET_BITS);
+				} else {
+					e[k] = in_pairs[i];
+					part[k] = (e[k].x >> PART_SLAB_BITS) & (PART_BUCKET_SLABS - 1u);
+				}
+			}
+		}
+		#pragma unroll
+		for (uint32_t k = 0; k < PART_PER_THREAD; ++k) if (part[k] != NONE) atomicAdd(&hist[part[k]], 1u);
+		__syncthreads();
+		// the chunk's share of every part's positions; where the parts start in the staged order
+		if (threadIdx.x < n_parts) {
+			const uint32_t v = hist[threadIdx.x];
+			uint32_t* cursor = LEVEL == 1 ? T.bucket_cursor + threadIdx.x : T.slab_cursor + ((bucket << PART_BUCKET_BITS) + threadIdx.x);
+			gbase[threadIdx.x] = v ? atomicAdd(cursor, v) : 0u;
+		}
+		if (threadIdx.x < 64u) {      // exclusive scan of the 256 counts (those past n_parts are zero): four a lane, then across the wavefront
+			const uint32_t d0 = threadIdx.x * 4u;
+			const uint32_t h0 = hist[d0], h1 = hist[d0 + 1u], h2 = hist[d0 + 2u], h3 = hist[d0 + 3u];
+			const uint32_t mine = h0 + h1 + h2 + h3;
+			uint32_t incl = mine;
+			#pragma unroll
+			for (uint32_t step = 1; step < 64u; step <<= 1) { const uint32_t up = __shfl_up(incl, step); if (threadIdx.x >= step) incl += up; }
+			const uint32_t before = incl - mine;
+			lstart[d0] = before; lstart[d0 + 1u] = before + h0; lstart[d0 + 2u] = before + h0 + h1; lstart[d0 + 3u] = before + h0 + h1 + h2;
+			if (threadIdx.x == 63u) lstart[PART_MAX_BUCKETS] = incl;
+		}
+		__syncthreads();
+		#pragma unroll
+		for (uint32_t k = 0; k < PART_PER_THREAD; ++k) if (part[k] != NONE) stage[lstart[part[k]] + atomicAdd(&fill[part[k]], 1u)] = e[k];
+		__syncthreads();
+		const uint32_t staged = lstart[PART_MAX_BUCKETS];
+		for (uint32_t j = threadIdx.x; j < staged; j += PART_PASS_THREADS) {
+			const U2 v = stage[j];
+			const uint32_t d = LEVEL == 1 ? v.x >> (PART_SLAB_BITS + PART_BUCKET_BITS) : (v.x >> PART_SLAB_BITS) & (PART_BUCKET_SLABS - 1u);
+			out_pairs[gbase[d] + (j - lstart[d])] = v;
+		}
+		__syncthreads();
+	}
+}
+
+// EMA: also apply k_ema_grid's decayed maximum to the slab's cells of the grid.  MERGE: the cells already hold another splat.
+template <bool EMA, bool MERGE>
+__global__ void __launch_bounds__(PART_THREADS) k_part_slabs(uint32_t n_total, const uint32_t* __restrict__ starts, const U2* __restrict__ pairs,
+                                                             uint32_t* __restrict__ grid_current_bits, float decay, float* __restrict__ grid) {
+	extern __shared__ uint32_t part_h[];      // the slab's cells
+	const uint32_t slab = blockIdx.x;
+	for (uint32_t j = threadIdx.x; j < PART_SLAB_CELLS; j += PART_THREADS) part_h[j] = 0u;
+	__syncthreads();
+	const uint32_t lo = starts[slab], hi = starts[slab + 1];
+	for (uint32_t i = lo + threadIdx.x; i < hi; i += PART_THREADS) {
+		const U2 e = pairs[i];
+		if (e.y) atomicMax(&part_h[e.x & (PART_SLAB_CELLS - 1u)], e.y);      // a zero cannot raise a cell
+	}
+	__syncthreads();
+	const uint32_t first = slab << PART_SLAB_BITS;
+	for (uint32_t j = threadIdx.x * 4u; j < PART_SLAB_CELLS; j += PART_THREADS * 4u) {
+		if (first + j + 3u < n_total) {
+			uint4 c = *(const uint4*)(part_h + j);
+			if (MERGE) {
+				const uint4 o = *(const uint4*)(grid_current_bits + first + j);
+				c.x = o.x > c.x ? o.x : c.x; c.y = o.y > c.y ? o.y : c.y; c.z = o.z > c.z ? o.z : c.z; c.w = o.w > c.w ? o.w : c.w;
+			}
+			*(uint4*)(grid_current_bits + first + j) = c;
+			if (EMA) {
+				float4 g = *(const float4*)(grid + first + j);
+				g.x = (g.x < 0.f) ? g.x : srf_max(g.x * decay, srf_u2f(c.x));
+				g.y = (g.y < 0.f) ? g.y : srf_max(g.y * decay, srf_u2f(c.y));
+				g.z = (g.z < 0.f) ? g.z : srf_max(g.z * decay, srf_u2f(c.z));
+				g.w = (g.w < 0.f) ? g.w : srf_max(g.w * decay, srf_u2f(c.w));
+				*(float4*)(grid + first + j) = g;
+			}
+		} else {
+			for (uint32_t k = 0; k < 4u && first + j + k < n_total; ++k) {
+				uint32_t c = part_h[j + k];
+				if (MERGE) { const uint32_t o = grid_current_bits[first + j + k]; c = o > c ? o : c; }
+				grid_current_bits[first + j + k] = c;
+				if (EMA) { const float g = grid[first + j + k]; grid[first + j + k] = (g < 0.f) ? g : srf_max(g * decay, srf_u2f(c)); }
+			}
+		}
+	}
+}
+
 // The splat of samples that arrive dealt by cell (k_generate_grid_samples_by_cell's order, taken as it is by the caller):
 // entry t = m n_cells + v lies in cell (v + 96925573) mod n_cells of some cascade when its point's first try passed, as nearly
 // all tries against the -0.01 threshold do.  A workgroup owns DEALT_CELLS consecutive cells of every cascade, reads the entries
@@ -517,6 +705,7 @@ int srf_sampler_create(const srf_sampler_config* c, srf_sampler_t** out) {
 	{ const char* v = getenv("SRF_MARCH_SKIP"); s->skip_enabled = !(v && v[0] == '0'); }
 	auto tri_state = [](const char* name) { const char* v = getenv(name); return v && v[0] == '0' ? 0 : (v && v[0] == '1' ? 1 : -1); };
 	s->force_splat_sort = tri_state("SRF_SPLAT_SORT");
+	{ const char* v = getenv("SRF_SPLAT_SORT"); if (v && v[0] == '2') s->force_splat_sort = 2; }      // 2: large-batch path through the library's sort
 	s->force_sample_bits = tri_state("SRF_GRID_SAMPLE_BITS");
 	s->force_sample_by_cell = tri_state("SRF_GRID_SAMPLE_BY_CELL");
 	s->count_probe_budget = COUNT_PROBE_BUDGET;
@@ -764,68 +953,133 @@ int srf_sampler_update_grid(srf_sampler_t* s, uint32_t n_total_positions, uint32
 	const void* rest_densities = grid_densities ? (const char*)grid_densities + (size_t)n_dealt * padded_output_width * (half ? 2 : 4) : nullptr;
 	bool sorted_splat = n >= SPLAT_SORT_MIN;
 	if (s->force_splat_sort >= 0) sorted_splat = s->force_splat_sort != 0 && n != 0;
-	// who clears the cells: the slabs of the sorted splat or the dealt splat, which write every cell, or else a fill
+	// large batches: the hand-made partition by slab; grids of more slabs than its histograms hold go through the library's sort
+	const uint32_t n_part_slabs = div_up(s->n_total, PART_SLAB_CELLS);
+	const bool partition = sorted_splat && n_part_slabs <= PART_MAX_SLABS && s->force_splat_sort != 2;
+	// who clears the cells: the dealt splat or the slabs of the sorted one, which write every cell, or else a fill
 	int rc = sorted_splat || n_dealt ? SRF_OK : fill_u32(s->density_grid_current, s->n_total, 0u, st);
 	if (rc != SRF_OK) return rc;
 	int end_bit = (int)SPLAT_SLAB_BITS + 1;
 	while (end_bit < 32 && (1ull << end_bit) < (unsigned long long)s->n_total) ++end_bit;
 	size_t temp_bytes = 0;
-	if (sorted_splat)
+	if (sorted_splat && !partition)
 		SRF_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, (const uint32_t*)nullptr, (uint32_t*)nullptr, (const uint32_t*)nullptr, (uint32_t*)nullptr,
 		                                           (int)n, (int)SPLAT_SLAB_BITS, end_bit, st));
 	const size_t arr = sorted_splat ? align_up((size_t)n * 4, 256) : 0;
-	const size_t sort_bytes = sorted_splat ? align_up(3 * arr + temp_bytes, 256) : 0;
+	const size_t part_words = align_up(((size_t)3 * n_part_slabs + 1 + 2 * PART_MAX_BUCKETS + 1) * 4, 256);
+	const size_t sort_bytes = !sorted_splat ? 0 : partition ? part_words + 2 * align_up((size_t)n, 32) * sizeof(U2) : align_up(3 * arr + temp_bytes, 256);
 	const size_t list_bytes = n_dealt ? 256 + (size_t)n_dealt * sizeof(U2) : 0;
 	rc = s->ws.reserve(sort_bytes + list_bytes);
 	if (rc != SRF_OK) return rc;
-	if (sorted_splat) {
-		uint32_t* thick = (uint32_t*)s->ws.ptr;
-		uint32_t* cells_sorted = (uint32_t*)((char*)s->ws.ptr + arr);
-		uint32_t* thick_sorted = (uint32_t*)((char*)s->ws.ptr + 2 * arr);
-		void* temp = (char*)s->ws.ptr + 3 * arr;
-		if (half)
-			hipLaunchKernelGGL(k_splat_values<true>, dim3(div_up(n, 256)), dim3(256), 0, st, n, padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, thick);
-		else
-			hipLaunchKernelGGL(k_splat_values<false>, dim3(div_up(n, 256)), dim3(256), 0, st, n, padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, thick);
-		SRF_LAUNCH_CHECK();
-		SRF_HIP(hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, rest_indices, cells_sorted, (const uint32_t*)thick, thick_sorted, (int)n, (int)SPLAT_SLAB_BITS, end_bit, st));
-		hipLaunchKernelGGL(k_splat_slabs, dim3(div_up(s->n_total, SPLAT_SLAB_CELLS)), dim3(256), 0, st, n, s->n_total, (const uint32_t*)cells_sorted,
-		                   (const uint32_t*)thick_sorted, (uint32_t*)s->density_grid_current);
-		SRF_LAUNCH_CHECK();
-	}
 	uint32_t* list_count = (uint32_t*)((char*)s->ws.ptr + sort_bytes);
 	U2* list = (U2*)((char*)s->ws.ptr + sort_bytes + 256);
-	if (n_dealt) {
-		rc = fill_u32(list_count, 1, 0u, st);
-		if (rc != SRF_OK) return rc;
+	bool ema_done = false;
+	// the dealt entries first where the partition follows: its slabs then merge with what is there and finish the update
+	auto dealt_splat = [&](bool merge) -> int {
+		int rc2 = fill_u32(list_count, 1, 0u, st);
+		if (rc2 != SRF_OK) return rc2;
 		uint32_t log2_cells = 0;
 		while ((1u << log2_cells) < nc) ++log2_cells;
 		const dim3 grid(nc / DEALT_CELLS), block(256);
 		const size_t lds = (size_t)s->P.n_cascades * DEALT_CELLS * sizeof(uint32_t);
 #define SRF_DEALT(H, M) hipLaunchKernelGGL((k_splat_dealt<H, M>), grid, block, lds, st, nc, log2_cells, s->P.n_cascades, n_dealt / nc, grid_indices, padded_output_width, grid_densities, \
                                            density_activation, s->P.min_cone_stepsize, (uint32_t*)s->density_grid_current, list_count, list)
-		if (half) { if (sorted_splat) SRF_DEALT(true, true); else SRF_DEALT(true, false); }
-		else { if (sorted_splat) SRF_DEALT(false, true); else SRF_DEALT(false, false); }
+		if (half) { if (merge) SRF_DEALT(true, true); else SRF_DEALT(true, false); }
+		else { if (merge) SRF_DEALT(false, true); else SRF_DEALT(false, false); }
 #undef SRF_DEALT
 		SRF_LAUNCH_CHECK();
-	}
-	if (!sorted_splat && n) {
-		if (half)
-			hipLaunchKernelGGL(k_splat_grid_samples<true>, dim3(div_up(n, 256)), dim3(256), 0, st, n, rest_indices,
-			                   padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, s->density_grid_current);
-		else
-			hipLaunchKernelGGL(k_splat_grid_samples<false>, dim3(div_up(n, 256)), dim3(256), 0, st, n, rest_indices,
-			                   padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, s->density_grid_current);
-		SRF_LAUNCH_CHECK();
-	}
-	if (n_dealt) {
+		return SRF_OK;
+	};
+	auto listed_splat = [&]() -> int {
 		hipLaunchKernelGGL(k_splat_listed, dim3(1024), dim3(256), 0, st, (const uint32_t*)list_count, (const U2*)list, s->n_total, (uint32_t*)s->density_grid_current);
 		SRF_LAUNCH_CHECK();
+		return SRF_OK;
+	};
+	if (partition) {
+		if (n_dealt) {
+			rc = dealt_splat(false);
+			if (rc == SRF_OK) rc = listed_splat();
+			if (rc != SRF_OK) return rc;
+		}
+		const uint32_t n_buckets = div_up(n_part_slabs, PART_BUCKET_SLABS);
+		uint32_t* counts = (uint32_t*)s->ws.ptr;
+		PartTables T;
+		T.starts = counts + n_part_slabs;
+		T.slab_cursor = T.starts + n_part_slabs + 1;
+		T.bucket_cursor = T.slab_cursor + n_part_slabs;
+		T.chunk_first = T.bucket_cursor + PART_MAX_BUCKETS;
+		const uint32_t* starts = T.starts;
+		U2* pairs_a = (U2*)((char*)s->ws.ptr + part_words);
+		U2* pairs = pairs_a + align_up((size_t)n, 32);
+		rc = fill_u32(counts, n_part_slabs, 0u, st);
+		if (rc != SRF_OK) return rc;
+		int dev = 0, n_cu = 0;
+		SRF_HIP(hipGetDevice(&dev));
+		SRF_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+		uint32_t groups = (uint32_t)n_cu * 2u;               // two workgroups of 1024 threads fill a CU
+		if (groups > div_up(n, PART_THREADS * 16u)) groups = div_up(n, PART_THREADS * 16u);
+		hipLaunchKernelGGL(k_part_count, dim3(groups), dim3(PART_THREADS), (size_t)n_part_slabs * sizeof(uint32_t), st, n, rest_indices, s->n_total, n_part_slabs, counts);
+		SRF_LAUNCH_CHECK();
+		hipLaunchKernelGGL(k_part_scan, dim3(1), dim3(PART_THREADS), 0, st, n_part_slabs, n_buckets, (const uint32_t*)counts, T);
+		SRF_LAUNCH_CHECK();
+		const uint32_t n_chunks = div_up(n, PART_CHUNK);
+		const uint32_t pass_groups = n_chunks + n_buckets < (uint32_t)n_cu * 8u ? n_chunks + n_buckets : (uint32_t)n_cu * 8u;      // pass 2 has at most n_chunks + n_buckets chunks
+#define SRF_PART_PASS(L, H) hipLaunchKernelGGL((k_part_pass<L, H>), dim3(pass_groups), dim3(PART_PASS_THREADS), 0, st, n, rest_indices, padded_output_width, rest_densities, \
+                                               density_activation, s->P.min_cone_stepsize, s->n_total, n_part_slabs, n_buckets, T, (const U2*)pairs_a, L == 1 ? pairs_a : pairs)
+		if (half) SRF_PART_PASS(1, true); else SRF_PART_PASS(1, false);
+		SRF_LAUNCH_CHECK();
+		SRF_PART_PASS(2, false);
+		SRF_LAUNCH_CHECK();
+#undef SRF_PART_PASS
+		const size_t slab_lds = (size_t)PART_SLAB_CELLS * sizeof(uint32_t);
+		if (n_dealt)
+			hipLaunchKernelGGL((k_part_slabs<true, true>), dim3(n_part_slabs), dim3(PART_THREADS), slab_lds, st, s->n_total, (const uint32_t*)starts, (const U2*)pairs,
+			                   (uint32_t*)s->density_grid_current, s->P.ema_decay, s->density_grid);
+		else
+			hipLaunchKernelGGL((k_part_slabs<true, false>), dim3(n_part_slabs), dim3(PART_THREADS), slab_lds, st, s->n_total, (const uint32_t*)starts, (const U2*)pairs,
+			                   (uint32_t*)s->density_grid_current, s->P.ema_decay, s->density_grid);
+		SRF_LAUNCH_CHECK();
+		ema_done = true;
+	} else {
+		if (sorted_splat) {
+			uint32_t* thick = (uint32_t*)s->ws.ptr;
+			uint32_t* cells_sorted = (uint32_t*)((char*)s->ws.ptr + arr);
+			uint32_t* thick_sorted = (uint32_t*)((char*)s->ws.ptr + 2 * arr);
+			void* temp = (char*)s->ws.ptr + 3 * arr;
+			if (half)
+				hipLaunchKernelGGL(k_splat_values<true>, dim3(div_up(n, 256)), dim3(256), 0, st, n, padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, thick);
+			else
+				hipLaunchKernelGGL(k_splat_values<false>, dim3(div_up(n, 256)), dim3(256), 0, st, n, padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, thick);
+			SRF_LAUNCH_CHECK();
+			SRF_HIP(hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, rest_indices, cells_sorted, (const uint32_t*)thick, thick_sorted, (int)n, (int)SPLAT_SLAB_BITS, end_bit, st));
+			hipLaunchKernelGGL(k_splat_slabs, dim3(div_up(s->n_total, SPLAT_SLAB_CELLS)), dim3(256), 0, st, n, s->n_total, (const uint32_t*)cells_sorted,
+			                   (const uint32_t*)thick_sorted, (uint32_t*)s->density_grid_current);
+			SRF_LAUNCH_CHECK();
+		}
+		if (n_dealt) {
+			rc = dealt_splat(sorted_splat);
+			if (rc != SRF_OK) return rc;
+		}
+		if (!sorted_splat && n) {
+			if (half)
+				hipLaunchKernelGGL(k_splat_grid_samples<true>, dim3(div_up(n, 256)), dim3(256), 0, st, n, rest_indices,
+				                   padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, s->density_grid_current);
+			else
+				hipLaunchKernelGGL(k_splat_grid_samples<false>, dim3(div_up(n, 256)), dim3(256), 0, st, n, rest_indices,
+				                   padded_output_width, rest_densities, density_activation, s->P.min_cone_stepsize, s->density_grid_current);
+			SRF_LAUNCH_CHECK();
+		}
+		if (n_dealt) {
+			rc = listed_splat();
+			if (rc != SRF_OK) return rc;
+		}
 	}
-	const uint32_t n_vec4 = s->n_total / 4;
-	const uint32_t blocks = div_up(n_vec4, 256) < 8192 ? div_up(n_vec4, 256) : 8192;
-	hipLaunchKernelGGL(k_ema_grid, dim3(blocks), dim3(256), 0, st, n_vec4, (const float4*)s->density_grid_current, s->P.ema_decay, (float4*)s->density_grid);
-	SRF_LAUNCH_CHECK();
+	if (!ema_done) {
+		const uint32_t n_vec4 = s->n_total / 4;
+		const uint32_t blocks = div_up(n_vec4, 256) < 8192 ? div_up(n_vec4, 256) : 8192;
+		hipLaunchKernelGGL(k_ema_grid, dim3(blocks), dim3(256), 0, st, n_vec4, (const float4*)s->density_grid_current, s->P.ema_decay, (float4*)s->density_grid);
+		SRF_LAUNCH_CHECK();
+	}
 	++s->i_step;
 	return SRF_OK;
 }

@@ -56,7 +56,8 @@ struct srf_sampler {
 	bool     skip_valid;    // skip_dist matches the bitfield
 	bool     skip_enabled;  // SRF_MARCH_SKIP=0 in the environment at creation switches the table off
 	// Switches the tests use to run both sides of a size-dependent choice on small inputs; read from the environment once, when the
-	// sampler is created (-1: the library chooses): SRF_SPLAT_SORT, SRF_GRID_SAMPLE_BITS, SRF_GRID_SAMPLE_BY_CELL = 0|1;
+	// sampler is created (-1: the library chooses): SRF_SPLAT_SORT, SRF_GRID_SAMPLE_BITS, SRF_GRID_SAMPLE_BY_CELL = 0|1
+	// (SRF_SPLAT_SORT=2: the large-batch splat through the library's radix sort instead of the partition made for it);
 	// SRF_COUNT_PROBE_BUDGET = lookups after which the counting march parks a ray (0: never)
 	int      force_splat_sort, force_sample_bits, force_sample_by_cell;
 	uint32_t count_probe_budget;

@@ -71,7 +71,7 @@ def test_device_reciprocal_is_the_ieee_quotient_for_every_mantissa(gpu):
 # the two forms of the grid update's heavy steps: lookups in the grid itself and device atomics per sample (what small
 # batches get), and the forms that large batches take, forced here on small ones (lookups in bit tables of the two
 # comparisons, points dealt to threads in the order of their candidate cells; samples sorted by slab of cells and combined in LDS)
-@pytest.mark.parametrize("large_batch_path", ["0", "1"])
+@pytest.mark.parametrize("large_batch_path", ["0", "1", "2"])       # direct atomics, the partition by slab, the library's sort
 @pytest.mark.parametrize("N,C", [((8, 8, 8), 1), ((16, 8, 8), 3), ((64, 32, 32), 5), ((128, 128, 128), 2)])
 def test_grid_maintenance(gpu, orc, N, C, large_batch_path, monkeypatch):
     torch = gpu
@@ -109,6 +109,7 @@ def test_grid_maintenance(gpu, orc, N, C, large_batch_path, monkeypatch):
         s.update_grid(n, 1, torch.from_numpy(dens).cuda(), idx, api.ACT_NONE)
         cur = np.zeros(n_total, np.float32)
         orc.splat_grid_samples(p, np.concatenate([wi1, wi2]), 1, dens, O.ACT_NONE, cur)
+        assert np.array_equal(s.density_grid_current.cpu().numpy(), cur)       # the public member the splat leaves (occupancy_sampler.h:118)
         orc.ema_grid(cur, p.ema_decay, o_grid)
         assert np.array_equal(s.density_grid.cpu().numpy(), o_grid)
         s.update_grid_bitfield()
