@@ -501,6 +501,44 @@ SRF_HD ShortChain short_chain_next(const ShortForm& f, const ShortChain& ch) {
 	return n;
 }
 
+// Many steps at once.  For a float g whose mantissa is below sqrt 2 the reciprocal of its reciprocal (both correctly rounded) is g
+// itself (every such mantissa checked: tests/test_disparity_chain.py), so while g = c + r stays in that lower part of a binade
+// [B, 2B) the reciprocal the chain carries is g and a step is the addition r <- c + r.  In one binade the floats are the
+// multiples m u of u = 2^-23 B, and c + r rounds to (m - q) u with q = |c| / u rounded to the nearest integer: the same q at every
+// step, unless |c| / u lies exactly halfway between two integers (the rounding then goes by m's parity).  The loop
+//     do r = c + r; while (r > S);
+// entered with r > S, therefore runs k = ceil((m - s) / q) times (S = s u, rounded down) and ends at (m - k q) u.
+// Asked of the caller: c < 0, r > S, both in the binade whose lowest value is `bin`, S >= (bin - c) (1 + 2^-22) so that the last sum
+// still lies in it, and c + r below sqrt 2 * bin.  Returns k with r moved there, or 0 with r untouched where the closed form
+// does not hold (the halfway case, a q the mantissa arithmetic does not cover, operands in different binades).
+SRF_HD uint32_t short_chain_jump(float c, float bin, float S, float& r) {
+	const uint32_t rb = srf_f2u(r), sb = srf_f2u(S), eb = srf_f2u(bin);
+	if ((rb & 0x7f800000u) != eb || (sb & 0x7f800000u) != eb || eb < (25u << 23)) return 0u;
+	const float inv_u = srf_u2f(((254u + 23u) << 23) - eb);      // 1 / u = 2^23 / bin
+	const float cu = -c * inv_u;                                    // |c| in units of u: exact (a power of two times c)
+	if (!(cu >= 1.0f && cu < 4194304.0f)) return 0u;
+	const float whole = __builtin_floorf(cu), part = cu - whole;    // below 2^22 a float has at least one fractional bit: part is exact
+	if (part == 0.5f) return 0u;
+	const uint32_t q = (uint32_t)whole + (part > 0.5f ? 1u : 0u);
+	const uint32_t m = (rb & 0x007fffffu) | 0x00800000u, s_int = (sb & 0x007fffffu) | 0x00800000u;
+	const uint32_t a = m - s_int;                                   // > 0: r > S
+	uint32_t k = (uint32_t)((float)a * srf_approx_rcp((float)q));   // a / q to within a few units, then made exact
+	while (k * q < a) ++k;
+	while (k > 1u && (k - 1u) * q >= a) --k;
+	if (k == 0u) k = 1u;
+	const uint32_t m_end = m - k * q;
+	if (k * q >= m || m_end < 0x00800000u) return 0u;              // (the caller's S rules this out)
+	r = srf_u2f(eb | (m_end & 0x007fffffu));
+	return k;
+}
+
+// does any lane of the wavefront that is executing this (on the host: the one caller) hold the condition?
+#if defined(__HIP_DEVICE_COMPILE__)
+#define SRF_WAVE_ANY(p) (__ballot(p) != 0ull)
+#else
+#define SRF_WAVE_ANY(p) (p)
+#endif
+
 template <uint32_t K>
 SRF_HD void count_steps(CountLane& L, const Params& P, const CountArgs& A) {
 	{
@@ -514,16 +552,39 @@ SRF_HD void count_steps(CountLane& L, const Params& P, const CountArgs& A) {
 			uint32_t n = 0;
 			const float lim = srf_min(L.t_limit, t_hi);
 			bool go = (t >= t_lo) & (t < lim);
+			{
+				// the stretch's steps inside the lower part of a binade, all at once (short_chain_jump); what is left (the upper
+				// part, the last few steps before the limit, the cases the closed form leaves out) goes through the burst below
+				const float g1 = f.c + ch.r;
+				const float bin = srf_u2f(srf_f2u(ch.r) & 0x7f800000u);
+				const float G = srf_approx_rcp(lim) * 1.000001f;      // r > G implies RN(1/r) < lim (see march_steps)
+				const float S = srf_max(G, (bin - f.c) * 1.0000002f);
+				if (go & (g1 >= bin) & (g1 < bin * 1.4142134f) & (ch.r > S)) {
+					float r = ch.r;
+					const uint32_t taken = short_chain_jump(f.c, bin, S, r);
+					if (taken) {
+						ch.r = r;
+						ch.t = srf_rcp_normal(r);
+						t = ch.t;
+						n = taken;
+						go = t < lim;
+					}
+				}
+			}
+			// in groups of four; the wavefront leaves as soon as none of its stepping lanes has a step left (after a jump most have not)
+			for (uint32_t k0 = 0; k0 < K; k0 += 4u) {
+				if (!SRF_WAVE_ANY(go)) break;
 #if defined(__HIP_DEVICE_COMPILE__)
-			#pragma unroll
+				#pragma unroll
 #endif
-			for (uint32_t k = 0; k < K; ++k) {
-				ch = short_chain_next(f, ch);      // a lane that has stopped runs on idle: its chain is not looked at again
-				const bool ok = go;
-				const float tn = ch.t;
-				t = ok ? tn : t;
-				n += ok ? 1u : 0u;
-				go = ok & (tn < lim);
+				for (uint32_t k = 0; k < 4u; ++k) {
+					ch = short_chain_next(f, ch);      // a lane that has stopped runs on idle: its chain is not looked at again
+					const bool ok = go;
+					const float tn = ch.t;
+					t = ok ? tn : t;
+					n += ok ? 1u : 0u;
+					go = ok & (tn < lim);
+				}
 			}
 			L.t = t;
 			L.step += n;
@@ -927,7 +988,7 @@ SRF_HD MarchEnd march_steps(MarchLane& L, const Params& P) {
 					const float S = srf_max(G, (bin - f.c) * 1.0000002f);
 					float r = ch.r;
 					if (r > S) {
-						do r = f.c + r; while (r > S);
+						if (!short_chain_jump(f.c, bin, S, r)) do r = f.c + r; while (r > S);
 						ch.r = r;
 						ch.t = srf_rcp_normal(r);
 					} else {

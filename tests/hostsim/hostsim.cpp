@@ -624,6 +624,41 @@ uint32_t hs_carried_reciprocal_failures() {
 	return fails;
 }
 
+// short_chain_jump against the loop of additions it stands for, on random operands of every kind the marches can hand it
+// (any binade, c from a few to millions of units of the binade's spacing, S anywhere between the lowest admissible value and r):
+// out[0] = cases where the closed form applied, out[1] = cases it declined, return = cases where count or end value differ
+uint32_t hs_chain_jump_mismatches(uint32_t seed, uint32_t n_cases, uint32_t* out) {
+	uint64_t state = 0x9e3779b97f4a7c15ull * (seed + 1);
+	auto next = [&]() { state = state * 6364136223846793005ull + 1442695040888963407ull; return (uint32_t)(state >> 33); };
+	uint32_t bad = 0;
+	out[0] = out[1] = 0;
+	for (uint32_t it = 0; it < n_cases; ++it) {
+		const uint32_t e = 40u + next() % 170u;                                  // binade
+		const float bin = srf_u2f(e << 23);
+		const uint32_t m = 0x00800000u | (next() & 0x007fffffu);
+		float r = srf_u2f((e << 23) | (m & 0x007fffffu));
+		// |c|: 1.5 .. 2^21 spacings, with a random mantissa; one case in eight exactly halfway between two multiples
+		const uint32_t units = 2u + next() % (1u << (1 + next() % 21));
+		float c = -(float)units * srf_u2f((e - 23u) << 23);
+		if ((next() & 7u) == 0u) c -= 0.5f * srf_u2f((e - 23u) << 23);
+		else c *= 1.0f + (float)(next() & 0xffffu) * (1.0f / 16777216.0f);
+		const float S_lo = (bin - c) * 1.0000002f;
+		if (!(r > S_lo) || (!(c + r < bin * 1.4142134f) && (next() & 1u))) continue;
+		float S = S_lo + (r - S_lo) * ((float)(next() & 0xffffu) / 65536.0f);
+		if (!(S >= S_lo)) S = S_lo;
+		if (!(r > S)) continue;
+		float r_loop = r;
+		uint32_t k_loop = 0;
+		do { r_loop = c + r_loop; ++k_loop; } while (r_loop > S && k_loop < (1u << 24));
+		float r_jump = r;
+		const uint32_t k = short_chain_jump(c, bin, S, r_jump);
+		if (k == 0) { ++out[1]; if (srf_f2u(r_jump) != srf_f2u(r)) ++bad; continue; }
+		++out[0];
+		if (k != k_loop || srf_f2u(r_jump) != srf_f2u(r_loop)) ++bad;
+	}
+	return bad;
+}
+
 // n steps from t0 by calc_dt and by the short form (which stops where its range ends); returns the short form's step count
 uint32_t hs_disparity_chains(const orc_params* p, float t0, uint32_t n, float* t_calc, float* t_short) {
 	const Params P = to_params(p);

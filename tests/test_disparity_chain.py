@@ -44,6 +44,15 @@ def test_short_chain_is_the_chain_of_calc_dt(orc, hostsim, near, far, n_steps):
     assert covered > 40 * min(n_steps, 64) // 4
 
 
+def test_many_additions_at_once_equal_the_loop(hostsim):
+    """short_chain_jump (srf_bodies.h): the k additions r <- c + r that end at or below S, in closed form on the mantissas, against the
+    loop itself; operands over every binade and step size, including steps exactly halfway between two floats, which it must decline"""
+    hostsim.lib.hs_chain_jump_mismatches.restype = C.c_uint32
+    out = (C.c_uint32 * 2)()
+    assert hostsim.lib.hs_chain_jump_mismatches(3, 400000, out) == 0
+    assert out[0] > 100000 and 1000 < out[1] < out[0]
+
+
 def test_wide_march_bookkeeping_matches_the_step_by_step_loop(hostsim):
     """wide_apply (64 steps of one ray at once, srf_bodies.h) against the loop of occupancy_sampler.cu:595-632 taken a step
     at a time, on random batches that include the exits the marches of the other tests rarely reach: the sample cap in
