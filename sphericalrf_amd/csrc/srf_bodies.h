@@ -165,7 +165,7 @@ SRF_HD bool mask_camera_sees(const float* m, Vec3 p, float radius, float focal_x
 // makes a wavefront wait for its unluckiest lane, a memory round trip per try.
 template <bool POW2, uint32_t BATCH>
 SRF_HD void grid_sample_tries_batched(uint32_t i, const Params& P, uint32_t n_elements, uint32_t step, uint32_t level, const float* grid_in, float thresh,
-                                      const uint32_t* above, uint32_t* cell_out, uint32_t* idx_out) {
+                                      const uint32_t* above, uint32_t* cell_out, uint32_t* idx_out, const uint32_t* above_summary = nullptr) {
 	static_assert(10 % BATCH == 0, "whole batches");
 	uint32_t cell = 0, idx = 0;
 	bool found = false;
@@ -180,7 +180,11 @@ SRF_HD void grid_sample_tries_batched(uint32_t i, const Params& P, uint32_t n_el
 			const uint32_t h = h0 + (j0 + q) * 19349663u;
 			c[q] = POW2 ? (h & (P.n_cells - 1u)) : (h % P.n_cells);
 			id[q] = c[q] + level * P.n_cells;
-			pass[q] = above ? ((above[id[q] >> 5] >> (id[q] & 31u)) & 1u) != 0u : grid_in[id[q]] > thresh;
+			// above_summary: one bit per word of `above`, set where the word has a cell that fails: a table small enough for the
+			// nearest cache, and where hardly any cell fails (the uniform draw: only masked cells do) it answers nearly every lookup
+			const uint32_t word = id[q] >> 5;
+			if (above_summary && ((above_summary[word >> 5] >> (word & 31u)) & 1u) == 0u) pass[q] = true;
+			else pass[q] = above ? ((above[word] >> (id[q] & 31u)) & 1u) != 0u : grid_in[id[q]] > thresh;
 		}
 #if defined(__HIP_DEVICE_COMPILE__)
 		#pragma unroll
@@ -194,11 +198,11 @@ SRF_HD void grid_sample_tries_batched(uint32_t i, const Params& P, uint32_t n_el
 }
 template <bool POW2>
 SRF_HD void grid_sample_tries(uint32_t i, const Params& P, uint32_t n_elements, uint32_t step, uint32_t level, const float* grid_in, float thresh,
-                              const uint32_t* above, uint32_t tries_at_once, uint32_t* cell_out, uint32_t* idx_out) {
-	if (tries_at_once >= 10u) grid_sample_tries_batched<POW2, 10>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out);
-	else if (tries_at_once >= 5u) grid_sample_tries_batched<POW2, 5>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out);
-	else if (tries_at_once >= 2u) grid_sample_tries_batched<POW2, 2>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out);
-	else grid_sample_tries_batched<POW2, 1>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out);
+                              const uint32_t* above, uint32_t tries_at_once, uint32_t* cell_out, uint32_t* idx_out, const uint32_t* above_summary = nullptr) {
+	if (tries_at_once >= 10u) grid_sample_tries_batched<POW2, 10>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out, above_summary);
+	else if (tries_at_once >= 5u) grid_sample_tries_batched<POW2, 5>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out, above_summary);
+	else if (tries_at_once >= 2u) grid_sample_tries_batched<POW2, 2>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out, above_summary);
+	else grid_sample_tries_batched<POW2, 1>(i, P, n_elements, step, level, grid_in, thresh, above, cell_out, idx_out, above_summary);
 }
 
 // above: optional table of the comparison grid_in[idx] > thresh, one bit per cell (bit idx & 31 of word idx >> 5),
@@ -206,7 +210,7 @@ SRF_HD void grid_sample_tries(uint32_t i, const Params& P, uint32_t n_elements, 
 SRF_HD void grid_sample_point(uint32_t i, const Params& P, uint32_t n_elements, Pcg32 rng, uint32_t step,
                               const float* grid_in, float thresh, Vec3* position, uint32_t* index, const uint32_t* above = nullptr,
                               const PcgSkip* skip = nullptr, uint32_t tries_at_once = 1,
-                             const uint64_t* skip16_m = nullptr, const uint64_t* skip16_p = nullptr) {
+                             const uint64_t* skip16_m = nullptr, const uint64_t* skip16_p = nullptr, const uint32_t* above_summary = nullptr) {
 	if (skip16_m) pcg_advance_skip16(rng, i * 4u, skip16_m, skip16_p);
 	else if (skip) pcg_advance_u32(rng, i * 4u, *skip);
 	else pcg_advance(rng, (uint64_t)(uint32_t)(i * 4u));
@@ -217,8 +221,8 @@ SRF_HD void grid_sample_point(uint32_t i, const Params& P, uint32_t n_elements, 
 	// an integer division costs some forty instructions, and there are up to ten here)
 	const bool pow2 = (P.n_cells & (P.n_cells - 1u)) == 0u;
 	uint32_t cell = 0, idx = 0;
-	if (pow2) grid_sample_tries<true>(i, P, n_elements, step, level, grid_in, thresh, above, tries_at_once, &cell, &idx);
-	else grid_sample_tries<false>(i, P, n_elements, step, level, grid_in, thresh, above, tries_at_once, &cell, &idx);
+	if (pow2) grid_sample_tries<true>(i, P, n_elements, step, level, grid_in, thresh, above, tries_at_once, &cell, &idx, above_summary);
+	else grid_sample_tries<false>(i, P, n_elements, step, level, grid_in, thresh, above, tries_at_once, &cell, &idx, above_summary);
 	const uint32_t x = morton3d_invert(cell), y = morton3d_invert(cell >> 1), z = morton3d_invert(cell >> 2);
 	const float jx = pcg_next_float(rng), jy = pcg_next_float(rng), jz = pcg_next_float(rng);
 	Vec3 pos = mk3(((float)x + jx) / (float)P.grid_size[0] - 0.5f, ((float)y + jy) / (float)P.grid_size[1] - 0.5f,
@@ -246,10 +250,10 @@ SRF_HD void grid_sample_point(uint32_t i, const Params& P, uint32_t n_elements, 
 SRF_HD void grid_sample_body(uint32_t i, const Params& P, uint32_t n_elements, Pcg32 rng, uint32_t step,
                              const float* grid_in, float thresh, float* positions, uint32_t* indices, const uint32_t* above = nullptr,
                              const PcgSkip* skip = nullptr, uint32_t tries_at_once = 1,
-                             const uint64_t* skip16_m = nullptr, const uint64_t* skip16_p = nullptr) {
+                             const uint64_t* skip16_m = nullptr, const uint64_t* skip16_p = nullptr, const uint32_t* above_summary = nullptr) {
 	Vec3 pos;
 	uint32_t idx;
-	grid_sample_point(i, P, n_elements, rng, step, grid_in, thresh, &pos, &idx, above, skip, tries_at_once, skip16_m, skip16_p);
+	grid_sample_point(i, P, n_elements, rng, step, grid_in, thresh, &pos, &idx, above, skip, tries_at_once, skip16_m, skip16_p, above_summary);
 	st3(positions + 3 * (size_t)i, pos);
 	indices[i] = idx;
 }

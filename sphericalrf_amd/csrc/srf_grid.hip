@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(256) k_mark_untrained(Params P, uint32_t n_tot
 __global__ void __launch_bounds__(256) k_generate_grid_samples(Params P, uint32_t n_elements, Pcg32 rng, uint32_t step,
                                                                 const float* __restrict__ grid_in, float thresh,
                                                                 float* __restrict__ positions, uint32_t* __restrict__ indices, const uint32_t* __restrict__ above,
-                                                                uint32_t tries_at_once, uint32_t first) {
+                                                                uint32_t tries_at_once, uint32_t first, const uint32_t* __restrict__ above_summary) {
 	// the generator's skip-ahead maps, one hexadecimal digit each, worked out once per workgroup
 	__shared__ uint64_t skip_m[128], skip_p[128];
 	if (threadIdx.x < 128) pcg_skip16_entry(rng, threadIdx.x, &skip_m[threadIdx.x], &skip_p[threadIdx.x]);
@@ -57,7 +57,7 @@ __global__ void __launch_bounds__(256) k_generate_grid_samples(Params P, uint32_
 	const uint32_t n_runs = (n_elements - first + 255u) / 256u;
 	for (uint32_t run = blockIdx.x; run < n_runs; run += gridDim.x) {
 		const uint32_t i = first + run * 256u + threadIdx.x;
-		if (i < n_elements) grid_sample_body(i, P, n_elements, rng, step, grid_in, thresh, positions, indices, above, nullptr, tries_at_once, skip_m, skip_p);
+		if (i < n_elements) grid_sample_body(i, P, n_elements, rng, step, grid_in, thresh, positions, indices, above, nullptr, tries_at_once, skip_m, skip_p, above_summary);
 	}
 }
 
@@ -134,16 +134,22 @@ __global__ void __launch_bounds__(256) k_grid_samples_to_point_order(uint32_t n_
 	indices[i] = srf_f2u(r.w);
 }
 
-// one bit per cell for each of two thresholds: bit (i & 31) of word (i >> 5) is grid[i] > thresh; 64 cells per wavefront round
+// one bit per cell for each of two thresholds: bit (i & 31) of word (i >> 5) is grid[i] > thresh; 64 cells per wavefront round.
+// summary_a (cleared by the caller): bit (w & 31) of word (w >> 5) is set where word w of above_a has a bit that is not set
 __global__ void __launch_bounds__(256) k_threshold_bits(const float* __restrict__ grid, uint32_t n_total, float thresh_a, float thresh_b,
-                                                         uint32_t* __restrict__ above_a, uint32_t* __restrict__ above_b) {
+                                                         uint32_t* __restrict__ above_a, uint32_t* __restrict__ above_b, uint32_t* __restrict__ summary_a) {
 	const uint32_t lane = threadIdx.x & 63u;
 	const uint32_t stride = gridDim.x * blockDim.x;
 	for (uint32_t base = (blockIdx.x * blockDim.x + threadIdx.x) - lane; base < n_total; base += stride) {   // uniform per wavefront
 		const uint32_t i = base + lane;
 		const float v = i < n_total ? grid[i] : 0.f;
 		const uint64_t ma = __ballot(i < n_total && v > thresh_a), mb = __ballot(i < n_total && v > thresh_b);
-		if (lane == 0) { above_a[base >> 5] = (uint32_t)ma; above_b[base >> 5] = (uint32_t)mb; }
+		if (lane == 0) {
+			above_a[base >> 5] = (uint32_t)ma; above_b[base >> 5] = (uint32_t)mb;
+			const uint32_t w = base >> 5;      // (even: both words of the round share a summary word)
+			const uint32_t some = ((uint32_t)ma != 0xffffffffu ? 1u : 0u) | ((uint32_t)(ma >> 32) != 0xffffffffu ? 2u : 0u);
+			if (some) atomicOr(&summary_a[w >> 5], some << (w & 31u));
+		}
 		if (lane == 32 && base + 32 < n_total) { above_a[(base >> 5) + 1] = (uint32_t)(ma >> 32); above_b[(base >> 5) + 1] = (uint32_t)(mb >> 32); }
 	}
 }
@@ -864,17 +870,23 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	const uint32_t n_dealt = cell_order ? n_uniform / nc * nc : 0u, n_dealt_b = cell_order ? n_nonuniform / nc * nc : 0u;
 	by_cell = by_cell && n_nonuniform > n_dealt_b;
 	const uint64_t dealt_threads = by_cell ? (uint64_t)div_up(n_nonuniform, nc) * nc - n_dealt_b : 0;       // those that go through the staging array
-	const int rc = s->ws.reserve(2 * table_bytes + dealt_threads * sizeof(Float4) + 256);
+	const size_t summary_words = tabulate ? div_up(div_up(s->n_total, 32), 32) + 1 : 0;
+	const size_t summary_bytes = align_up(summary_words * 4, 256);
+	int rc = s->ws.reserve(2 * table_bytes + summary_bytes + dealt_threads * sizeof(Float4) + 256);
 	if (rc != SRF_OK) return rc;
 	const uint32_t* above_a = nullptr;
 	const uint32_t* above_b = nullptr;
+	const uint32_t* summary_a = nullptr;
 	if (tabulate) {
 		uint32_t* a = (uint32_t*)s->ws.ptr;
 		uint32_t* b = (uint32_t*)((char*)s->ws.ptr + table_bytes);
+		uint32_t* sum = (uint32_t*)((char*)s->ws.ptr + 2 * table_bytes);
+		rc = fill_u32(sum, summary_words, 0u, st);
+		if (rc != SRF_OK) return rc;
 		const uint32_t blocks = div_up(s->n_total, 256) < 16384 ? div_up(s->n_total, 256) : 16384;
-		hipLaunchKernelGGL(k_threshold_bits, dim3(blocks), dim3(256), 0, st, (const float*)s->density_grid, s->n_total, -0.01f, s->P.min_optical_thickness, a, b);
+		hipLaunchKernelGGL(k_threshold_bits, dim3(blocks), dim3(256), 0, st, (const float*)s->density_grid, s->n_total, -0.01f, s->P.min_optical_thickness, a, b, sum);
 		SRF_LAUNCH_CHECK();
-		above_a = a; above_b = b;
+		above_a = a; above_b = b; summary_a = sum;
 	}
 	const uint32_t tries = 10;    // the second draw looks all ten candidates of a point up at once: most fail in a trained grid (168 M points: 9.5 -> 6.2 ms)
 	auto dealt_grid = [](uint32_t windows) { return windows < 16384u ? windows : 16384u; };
@@ -892,7 +904,7 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	if (n_uniform > n_dealt) {
 		const uint32_t runs = div_up(n_uniform - n_dealt, 256);
 		hipLaunchKernelGGL(k_generate_grid_samples, dim3(runs < 16384u ? runs : 16384u), dim3(256), 0, st, s->P, n_uniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, -0.01f, grid_positions, grid_indices, above_a, 1u, n_dealt);   // nearly every first try passes
+		                   (const float*)s->density_grid, -0.01f, grid_positions, grid_indices, above_a, 1u, n_dealt, summary_a);   // nearly every first try passes
 		SRF_LAUNCH_CHECK();
 	}
 	pcg_advance(s->rng, 1ull << 32);
@@ -904,7 +916,7 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 		SRF_LAUNCH_CHECK();
 	}
 	if (by_cell) {
-		Float4* staged = (Float4*)((char*)s->ws.ptr + 2 * table_bytes);
+		Float4* staged = (Float4*)((char*)s->ws.ptr + 2 * table_bytes + summary_bytes);
 		// the whole multiples of the cell count, then the one the points do not fill
 		const uint64_t full_threads = (uint64_t)n_nonuniform / nc * nc - n_dealt_b;
 		if (full_threads) {
@@ -925,7 +937,7 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 	} else if (n_nonuniform > n_dealt_b) {
 		const uint32_t runs = div_up(n_nonuniform - n_dealt_b, 256);
 		hipLaunchKernelGGL(k_generate_grid_samples, dim3(runs < 16384u ? runs : 16384u), dim3(256), 0, st, s->P, n_nonuniform, s->rng, s->i_step,
-		                   (const float*)s->density_grid, s->P.min_optical_thickness, positions_b, indices_b, above_b, tries, n_dealt_b);
+		                   (const float*)s->density_grid, s->P.min_optical_thickness, positions_b, indices_b, above_b, tries, n_dealt_b, (const uint32_t*)nullptr);
 		SRF_LAUNCH_CHECK();
 	}
 	pcg_advance(s->rng, 1ull << 32);
