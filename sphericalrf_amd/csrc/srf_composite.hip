@@ -636,15 +636,20 @@ static int check_chain_error(srf_marcher* m) {
 // must not exceed that.  Asked of the runtime once per kernel variant.
 template <bool HI, bool HO, bool PL>
 static int stream_resident_workgroups(uint32_t* out) {
-	static uint32_t cached = 0;   // per variant; the library drives one device per process
+	constexpr int MAX_DEVICES = 64;
+	static uint32_t per_device[MAX_DEVICES];      // per variant and device (racing first calls both write the same value)
+	int dev = 0;
+	SRF_HIP(hipGetDevice(&dev));
+	SRF_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "compositing: device index %d out of range", dev);
+	uint32_t cached = per_device[dev];
 	if (!cached) {
-		hipDeviceProp_t prop; int dev = 0, per_cu = 0;
-		SRF_HIP(hipGetDevice(&dev));
+		hipDeviceProp_t prop; int per_cu = 0;
 		SRF_HIP(hipGetDeviceProperties(&prop, dev));
 		SRF_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k_composite_stream<HI, HO, PL>, (int)STREAM_THREADS, 0));
 		if (per_cu < 1) SRF_FAIL(SRF_ERR_HIP, "compositing: the streaming kernel does not fit this device");
 		if (per_cu > (int)STREAM_WORKGROUPS_PER_CU) per_cu = (int)STREAM_WORKGROUPS_PER_CU;
 		cached = (uint32_t)prop.multiProcessorCount * (uint32_t)per_cu;
+		per_device[dev] = cached;
 	}
 	*out = cached;
 	return SRF_OK;
