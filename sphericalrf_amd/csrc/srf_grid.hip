@@ -224,7 +224,7 @@ constexpr uint32_t PART_BUCKET_SLABS = 1u << PART_BUCKET_BITS;
 constexpr uint32_t PART_MAX_BUCKETS = 256;
 constexpr uint32_t PART_MAX_SLABS = PART_MAX_BUCKETS * PART_BUCKET_SLABS;      // 16384 slabs = 2^28 cells
 constexpr uint32_t PART_THREADS = 1024;
-constexpr uint32_t PART_CHUNK = 8192, PART_PASS_THREADS = 512, PART_PER_THREAD = PART_CHUNK / PART_PASS_THREADS;
+constexpr uint32_t PART_CHUNK = 8192, PART_PASS_THREADS = 1024, PART_PER_THREAD = PART_CHUNK / PART_PASS_THREADS;
 
 __global__ void __launch_bounds__(PART_THREADS) k_part_count(uint32_t n, const uint32_t* __restrict__ indices, uint32_t n_total, uint32_t n_slabs, uint32_t* __restrict__ counts) {
 	extern __shared__ uint32_t part_h[];
