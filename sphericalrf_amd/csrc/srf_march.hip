@@ -13,10 +13,11 @@ namespace srf {
 // waiting for (stepping through known-empty space, probing the grid, or picking up the next ray
 // of the block's range), so the expensive probe is issued for many lanes at once instead of
 // whenever any single lane needs one.
-// steps per stepping round: long enough to spread the round's fixed work (phase ballots, the first reciprocal of the
-// chain, the exit checks) over many steps, short enough that lanes waiting for a probe are not held up (8: 2.17 ms,
-// 16: 1.91 ms, 24: 1.66 ms, 32: 1.68 ms, 48: 1.71 ms for the march of the 2^20-ray batch)
-constexpr uint32_t COUNT_STEP_BURST = 24;
+// steps per stepping round, at most: long enough to spread the round's fixed work (phase ballots, the first reciprocal of the
+// chain, the closed-form stretch) over many steps; the burst runs in groups of four and ends when no lane has a step left, so a
+// long limit costs the lanes that wait for a probe little (24: 1.51 ms, 32: 1.33 ms, 48: 1.29 ms, 64: 1.35 ms for the march of
+// the 2^20-ray batch, with probing lanes waiting until they outnumber the stepping ones 32 to 1)
+constexpr uint32_t COUNT_STEP_BURST = 48;
 
 // five wavefronts a SIMD: 102 registers a lane, which the counting march just fits
 #define SRF_COUNT_WAVES_PER_EU 5
@@ -538,8 +539,9 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 	if (probe_budget) hipLaunchKernelGGL(k_zero_word, dim3(1), dim3(1), 0, st, ca.parked_count);
 	// rays per wavefront: enough for lanes that finish early to pick up more work, few enough for several wavefronts per SIMD
 	// (settled by measurement on the 2^20-ray training batch: one ray a lane; a probe round once every lane waits for one or the stepping
-	// lanes are outnumbered 8 to 1; new rays are begun 32 at a time)
-	constexpr uint32_t rays_per_wave = 64, probe_quorum = 64, begin_quorum = 32, probe_ratio = 8;
+	// lanes are outnumbered 32 to 1 — 4: 1.52, 8: 1.41, 16: 1.33, 24: 1.30, 32: 1.29, 48: 1.31, 64: 1.37 ms; stepping rounds are cheap since
+	// whole stretches are taken in closed form, so the probes wait for nearly all of them; new rays are begun 32 at a time)
+	constexpr uint32_t rays_per_wave = 64, probe_quorum = 64, begin_quorum = 32, probe_ratio = 32;
 	const uint32_t* order = nullptr;
 	if (sort_rays) {
 		uint32_t* order_out = (uint32_t*)(w + off_order);
