@@ -182,16 +182,16 @@ def bench_training_step(torch, api, scene, steps, warmup, n_rays=1 << 20, cap=1 
                 n_max_steps=int(info.n_max_steps), workload=w, sampler=s, occupied_bits=occupied_bits)
 
 
-def cpu_baseline(result, n_rays_sample=1 << 16):
-    """the oracle on a slice of the same workload: the first n_rays_sample rays of a batch, march + compositing fwd/bwd"""
+def cpu_baseline(result, bf, n_rays_sample=1 << 16):
+    """the oracle on a slice of the same workload: the first n_rays_sample rays of a batch, march + compositing fwd/bwd;
+    bf: the workload's bitfield in host memory"""
     import numpy as np
     from oracle import oracle as O
     from oracle import support as helpers
     from oracle.support import loss_args
     orc = O.get()
-    w, s = result["workload"], result["sampler"]
+    w = result["workload"]
     p = helpers.oracle_params(orc, w["sampler"])
-    bf = s.density_grid_bitfield.cpu().numpy()
     ds = orc.make_dataset(w["cameras"], w["resolution"], w["focal"], (0.5, 0.5))
     cap = n_rays_sample * 32
     best = None
@@ -379,7 +379,8 @@ def main():
                      "algorithmic_bytes": COMPOSITE_BYTES_PER_SAMPLE * r["n_samples"] + COMPOSITE_BYTES_PER_RAY * r["n_kept"]},
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(r)
+        out["cpu_baseline"] = None      # (keeps its place in the line; measured last, so that the host threads it starts are not around while the GPU is timed)
+    bits_host = r["sampler"].density_grid_bitfield.cpu().numpy() if not args.no_cpu_baseline else None
     if not args.no_extras:
         extras = []
         del r["sampler"]
@@ -409,6 +410,8 @@ def main():
             del t
             torch.cuda.empty_cache()
         out["extras"] = extras
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(r, bits_host)
     print(json.dumps(out), flush=True)
 
 
