@@ -70,7 +70,7 @@ using WideGeometry = Geometry<256, 7, true>;
 using StreamGeometry = Geometry<384, 5, false>;
 
 constexpr uint32_t GAP_SLACK = 1024; // a group whose sample range exceeds its sample count by more takes the per-ray path
-constexpr uint32_t CHAIN_UNROLL = 4;
+constexpr uint32_t CHAIN_UNROLL = 8;
 constexpr uint32_t COUNT_UNROLL = 8;
 constexpr uint32_t NPLAN = 4;        // plans kept at once by a kernel that has three items under way and plans a fourth
 
