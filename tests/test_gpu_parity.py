@@ -121,6 +121,47 @@ def test_grid_maintenance(gpu, orc, N, C, large_batch_path, monkeypatch):
     assert s.i_step == 3
 
 
+@pytest.mark.parametrize("path", ["1", "2"])       # the partition by slab, the library's sort
+def test_update_grid_of_arbitrary_batches_through_the_large_batch_paths(gpu, orc, path, monkeypatch):
+    """update_grid on its own, fed batches that no sampler draw produces: one sample, sizes around the partition's chunk of 8192, every
+    sample in one cell, one slab left empty, four values a sample with fp32 densities and an Exponential activation, previous grid
+    values that are masked or larger than what arrives: `density_grid_current` and `density_grid` against the oracle's splat and decay
+    (occupancy_sampler.cu:187-238)"""
+    torch = gpu
+    monkeypatch.setenv("SRF_SPLAT_SORT", path)
+    from sphericalrf_amd import api
+    cfg = dict(warping_type="ERP", aabb_scale=16, grid_size=(64, 32, 32), num_cascades=5, grid_distribution_type="WarpedSpace_Exp", init_grid_with_mask=False,
+               maximum_marching_steps=256, sampling_type="Disparity", near_distance=0.05, far_distance=10.0)
+    p = helpers.oracle_params(orc, cfg)
+    s = api.OccupancySampler(cfg)
+    n_total = p.n_total                                   # 327,680 cells: 20 slabs of 16384
+    rng = np.random.default_rng(17)
+    o_grid = (rng.random(n_total) * 0.5).astype(np.float32)
+    o_grid[rng.random(n_total) < 0.1] = -1.0              # masked cells keep their value
+    s.set_density_grid(torch.from_numpy(o_grid).cuda())
+    cases = [(1, 1, np.float16, "spread"), (8191, 1, np.float16, "spread"), (8192, 4, np.float32, "spread"), (8193, 1, np.float16, "one_cell"),
+             (50000, 1, np.float16, "no_slab_3"), (1000003, 4, np.float16, "spread"), (300000, 1, np.float32, "hot_cells")]
+    for n, width, dtype, kind in cases:
+        if kind == "one_cell":
+            idx = np.full(n, 123457, np.uint32)
+        elif kind == "no_slab_3":
+            idx = rng.integers(0, n_total - 16384, n).astype(np.uint32)
+            idx[idx >= 3 * 16384] += 16384
+        elif kind == "hot_cells":
+            idx = (rng.integers(0, 64, n) * 5003).astype(np.uint32)
+        else:
+            idx = rng.integers(0, n_total, n).astype(np.uint32)
+        act = O.ACT_EXPONENTIAL if width == 4 else O.ACT_NONE
+        raw = rng.normal(size=(n, width)).astype(dtype) if act == O.ACT_EXPONENTIAL else np.log1p(np.exp(rng.normal(size=(n, width)))).astype(dtype)
+        raw[rng.random(n) < 0.2, 0] = -20.0 if act == O.ACT_EXPONENTIAL else 0.0      # samples that raise (next to) nothing
+        s.update_grid(n, width, torch.from_numpy(raw).cuda(), torch.from_numpy(idx.view(np.int32)).cuda(), act)
+        cur = np.zeros(n_total, np.float32)
+        orc.splat_grid_samples(p, idx, width, raw, act, cur)
+        orc.ema_grid(cur, p.ema_decay, o_grid)
+        assert np.array_equal(s.density_grid_current.cpu().numpy().view(np.uint32), cur.view(np.uint32)), (n, width, kind)
+        assert np.array_equal(s.density_grid.cpu().numpy().view(np.uint32), o_grid.view(np.uint32)), (n, width, kind)
+
+
 # The opt-in cell order of the uniform points: the entries are the reference's points in the documented permutation, and
 # update_grid, given densities and indices in that order, leaves the grid the oracle gets from the reference's order.
 # Step 0: every point in cell order (a whole multiple of the cell count).  Step 1: a grid with masked cells, so that some
