@@ -150,10 +150,84 @@ __global__ void __launch_bounds__(128) k_train_count_wide(Params P, CountArgs A)
 
 __global__ void k_zero_word(uint32_t* p) { *p = 0u; }
 
-__global__ void __launch_bounds__(256) k_train_keep(uint32_t n_rays, uint32_t n_coords, const uint32_t* __restrict__ counts,
-                                                    const uint32_t* __restrict__ base, uint32_t* __restrict__ keep) {
-	const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-	if (i < n_rays) keep[i] = train_keep_flag(counts[i], base[i], n_coords);
+// Sample offsets and ray indices of a training batch in three launches.  A ray's first sample is the sum of the counts of
+// all rays before it (occupancy_sampler.cu:634: the counter advances by every ray's count, kept or not); a ray is kept when
+// its samples fit (train_keep_flag); a kept ray's index is the number of kept rays before it.  Tiles of 1024 rays:
+//   k_train_tile_counts   count sum of every tile; copies the two counters' values at entry
+//   k_train_bases         a tile's first offset = entry value + the sums of the tiles before it (every workgroup adds them up
+//                         itself: 1024 words for 2^20 rays); offsets, keep flags, kept rays of the tile; new sample counter
+//   k_train_ray_indices   the same over the kept flags; new ray counter
+constexpr uint32_t OFFSET_THREADS = 256;
+constexpr uint32_t OFFSET_TILE = 1024;
+
+struct TrainOffsetScratch {
+	uint32_t* tile_counts;   // [n_tiles]
+	uint32_t* tile_kept;     // [n_tiles]
+	uint32_t* entry;         // [2]: sample counter, ray counter when the call began
+};
+
+static size_t train_offset_scratch_bytes(uint32_t n_rays) { return align_up(((size_t)div_up(n_rays ? n_rays : 1u, OFFSET_TILE) * 2 + 2) * sizeof(uint32_t), 256); }
+
+__global__ void __launch_bounds__(OFFSET_THREADS) k_train_tile_counts(uint32_t n_rays, const uint32_t* __restrict__ counts, TrainOffsetScratch S,
+                                                                      const uint32_t* __restrict__ n_coords_counter, const uint32_t* __restrict__ n_rays_counter) {
+	__shared__ uint32_t lds[OFFSET_THREADS / 64];
+	const uint32_t first = blockIdx.x * OFFSET_TILE + threadIdx.x * 4;
+	uint32_t v = 0;
+	for (uint32_t k = 0; k < 4; ++k) if (first + k < n_rays) v += counts[first + k];
+	const uint32_t total = block_sum_u32<OFFSET_THREADS>(v, lds);
+	if (threadIdx.x == 0) S.tile_counts[blockIdx.x] = total;
+	if (blockIdx.x == 0 && threadIdx.x == 0) { S.entry[0] = *n_coords_counter; S.entry[1] = *n_rays_counter; }
+}
+
+// sum of the tile sums before this workgroup's tile (wrapping, like the counter it continues)
+__device__ __forceinline__ uint32_t tiles_before(const uint32_t* __restrict__ tile_sums, uint32_t* lds) {
+	uint32_t v = 0;
+	for (uint32_t k = threadIdx.x; k < blockIdx.x; k += OFFSET_THREADS) v += tile_sums[k];
+	return block_sum_u32<OFFSET_THREADS>(v, lds);
+}
+
+__global__ void __launch_bounds__(OFFSET_THREADS) k_train_bases(uint32_t n_rays, uint32_t n_coords, const uint32_t* __restrict__ counts, TrainOffsetScratch S,
+                                                                uint32_t* __restrict__ base, uint32_t* __restrict__ keep, uint32_t* __restrict__ n_coords_counter) {
+	__shared__ uint32_t lds[OFFSET_THREADS / 64 + 1];
+	const uint32_t before = S.entry[0] + tiles_before(S.tile_counts, lds);
+	const uint32_t first = blockIdx.x * OFFSET_TILE + threadIdx.x * 4;
+	uint32_t c[4];
+	uint32_t sum = 0;
+	for (uint32_t k = 0; k < 4; ++k) { c[k] = first + k < n_rays ? counts[first + k] : 0u; sum += c[k]; }
+	uint32_t total;
+	uint32_t run = before + block_exclusive_scan_u32<OFFSET_THREADS>(sum, lds, &total);
+	uint32_t kept = 0;
+	for (uint32_t k = 0; k < 4; ++k) {
+		if (first + k < n_rays) {
+			const uint32_t flag = train_keep_flag(c[k], run, n_coords);
+			base[first + k] = run;
+			keep[first + k] = flag;
+			kept += flag;
+		}
+		run += c[k];
+	}
+	const uint32_t kept_total = block_sum_u32<OFFSET_THREADS>(kept, lds);
+	if (threadIdx.x == 0) {
+		S.tile_kept[blockIdx.x] = kept_total;
+		if (blockIdx.x + 1 == gridDim.x) *n_coords_counter = before + total;
+	}
+}
+
+__global__ void __launch_bounds__(OFFSET_THREADS) k_train_ray_indices(uint32_t n_rays, const uint32_t* __restrict__ keep, TrainOffsetScratch S,
+                                                                      uint32_t* __restrict__ ridx, uint32_t* __restrict__ n_rays_counter) {
+	__shared__ uint32_t lds[OFFSET_THREADS / 64 + 1];
+	const uint32_t before = S.entry[1] + tiles_before(S.tile_kept, lds);
+	const uint32_t first = blockIdx.x * OFFSET_TILE + threadIdx.x * 4;
+	uint32_t f[4];
+	uint32_t sum = 0;
+	for (uint32_t k = 0; k < 4; ++k) { f[k] = first + k < n_rays ? keep[first + k] : 0u; sum += f[k]; }
+	uint32_t total;
+	uint32_t run = before + block_exclusive_scan_u32<OFFSET_THREADS>(sum, lds, &total);
+	for (uint32_t k = 0; k < 4; ++k) {
+		if (first + k < n_rays) ridx[first + k] = run;
+		run += f[k];
+	}
+	if (threadIdx.x == 0 && blockIdx.x + 1 == gridDim.x) *n_rays_counter = before + total;
 }
 
 // Writing march, one wavefront per block.  The samples of the block's kept rays form one run of the sample arrays
@@ -497,7 +571,7 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 	// final clamp to the far plane); rays that take more steps fall back to a full second march
 	uint32_t log_words = s->P.use_grid ? (s->P.n_max_steps + 64 + 31) / 32 : 0;
 	if (log_words > LOG_MAX_WORDS) log_words = LOG_MAX_WORDS;
-	const size_t off_log = align_up(off_scan + scan_scratch_bytes(n_rays), 256);
+	const size_t off_log = align_up(off_scan + train_offset_scratch_bytes(n_rays), 256);
 	// marching order: chunks of rays sorted by (image, pixel tile)
 	constexpr bool sort_rays = true;
 	const size_t off_order = align_up(off_log + (size_t)log_words * n * 8, 256);
@@ -595,12 +669,13 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 		else hipLaunchKernelGGL(k_train_count_wide<false>, dim3(wide_blocks), dim3(128), 0, st, s->P, ca);
 		SRF_LAUNCH_CHECK();
 	}
-	rc = scan_exclusive_u32(counts, base, n_rays, n_coords_counter, n_coords_counter, scan, st);
-	if (rc != SRF_OK) return rc;
-	hipLaunchKernelGGL(k_train_keep, dim3(div_up(n_rays, 256)), dim3(256), 0, st, n_rays, n_coords, (const uint32_t*)counts, (const uint32_t*)base, keep);
+	const uint32_t n_tiles = div_up(n_rays, OFFSET_TILE);
+	TrainOffsetScratch os;
+	os.tile_counts = (uint32_t*)scan; os.tile_kept = os.tile_counts + n_tiles; os.entry = os.tile_kept + n_tiles;
+	hipLaunchKernelGGL(k_train_tile_counts, dim3(n_tiles), dim3(OFFSET_THREADS), 0, st, n_rays, (const uint32_t*)counts, os, (const uint32_t*)n_coords_counter, (const uint32_t*)n_rays_counter);
+	hipLaunchKernelGGL(k_train_bases, dim3(n_tiles), dim3(OFFSET_THREADS), 0, st, n_rays, n_coords, (const uint32_t*)counts, os, base, keep, n_coords_counter);
+	hipLaunchKernelGGL(k_train_ray_indices, dim3(n_tiles), dim3(OFFSET_THREADS), 0, st, n_rays, (const uint32_t*)keep, os, ridx, n_rays_counter);
 	SRF_LAUNCH_CHECK();
-	rc = scan_exclusive_u32(keep, ridx, n_rays, n_rays_counter, n_rays_counter, scan, st);
-	if (rc != SRF_OK) return rc;
 	hipLaunchKernelGGL(k_train_write, dim3(div_up(n_rays, 64)), dim3(64), 0, st, s->P, n_rays, ds, bitfield, (const TrainRay*)state,
 	                   (const uint32_t*)counts, (const uint32_t*)base, (const uint32_t*)keep, (const uint32_t*)ridx,
 	                   rays, rays_rgba, ray_coord_indices, coords, sample_t, sample_dt, sample_cell, log);
