@@ -253,8 +253,9 @@ int  srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const
  * The same call for callers that must not allocate device memory while they run (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It runs the single-launch implementation with its
  * scratch (the per-item status words, item lists and per-ray side array of the ordered-offset chain) in an array that is part of
- * the library's device image, about 1.3 MB on every GPU the library runs on, and calls no hipMalloc / hipFree.
- * Limits: n_rays <= SRF_NOALLOC_MAX_RAYS; no distortion regulariser; refused on a marcher that has left the streaming kernel
+ * the library's device image, about 1.8 MB on every GPU the library runs on, and calls no hipMalloc / hipFree.
+ * Limits: n_rays <= SRF_NOALLOC_MAX_RAYS; no distortion regulariser; 64 consecutive rays whose samples need more than eight of the
+ * kernel's windows of 1920 are composited on a slower path (same results); refused on a marcher that has left the streaming kernel
  * (after a failed chain, or created under SRF_COMPOSITE_IMPL).  All calls on one GPU, of whatever marcher, share the array and
  * the chain's error word in it: at most one such call may be in flight per GPU, and calls that overlap on one GPU (different
  * streams or threads) race.  Because the next call's preparation clears the shared error word, a marcher without a host-visible

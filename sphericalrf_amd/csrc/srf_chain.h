@@ -28,12 +28,14 @@ struct ChainScratch {
 	uint32_t* slow_count;               // number of entries of slow_items
 	uint32_t* n_items;                  // number of items
 	uint32_t* group_words;              // per group: how many items it makes (fused::group_items_word)
+	unsigned long long* group_cuts;     // per group that makes several: at which rays its items begin (fused::plan_cuts)
 	uint32_t* prepare_sums;             // per workgroup of k_chain_prepare: how many items its groups make
 	U2* items;                          // the items in ray order (fused::items_of_group)
 	uint32_t* slow_items;               // items of groups that the streaming path does not take (see k_chain_prepare)
 	uint32_t* side;                     // per ray of such a group: samples consumed (forward kernel), then compacted offset (streaming kernel)
 	uint32_t* host_error;               // like error, in host memory the device can write (may be NULL)
 	uint32_t spin_limit;                // polls an item makes before it gives up
+	uint32_t max_parts;                 // items a group may be cut into (what the scratch has room for)
 	// the wave-per-item kernel's words (these three are zero between calls: its last workgroup to leave clears them)
 	uint32_t* ticket;                   // rounds of items handed out so far
 	uint32_t* disorder;                 // set when the call's rays are not laid out in increasing order

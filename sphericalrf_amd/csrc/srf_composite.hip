@@ -44,25 +44,27 @@ __global__ void __launch_bounds__(128) k_volume_rendering(Params P, srf_render_a
 // ------------------------------------------------------------------------------------
 // Single-launch compositing (phases in srf_composite_fused.h)
 // ------------------------------------------------------------------------------------
-// bytes of device scratch the chain needs for n_rays rays, and where its parts lie (a group makes at most two items)
-struct ChainLayout { size_t off_seg, off_prefix, off_misc, off_words, off_sums, off_items, off_list, off_side, bytes; };
-SRF_HD constexpr ChainLayout chain_layout(uint32_t n_rays) {
+// bytes of device scratch the chain needs for n_rays rays whose groups are cut into at most max_parts items each, and where
+// its parts lie
+struct ChainLayout { size_t off_seg, off_prefix, off_misc, off_words, off_cuts, off_sums, off_items, off_list, off_side, bytes; };
+SRF_HD constexpr ChainLayout chain_layout(uint32_t n_rays, uint32_t max_parts) {
 	const size_t n_groups = ((size_t)n_rays + fused::RAYS - 1) / fused::RAYS;
-	const size_t n_items = 2 * n_groups;
+	const size_t n_items = (size_t)max_parts * n_groups;
 	ChainLayout L = {};
 	L.off_seg = (n_items * 8 + 255) / 256 * 256;
 	L.off_prefix = (L.off_seg + (n_items + 63) / 64 * 8 * SEG_STRIDE + 255) / 256 * 256;
 	L.off_misc = (L.off_prefix + (n_items + 63) / 64 * 8 + 255) / 256 * 256;
 	L.off_words = L.off_misc + 512;
-	L.off_sums = (L.off_words + n_groups * 4 + 255) / 256 * 256;
+	L.off_cuts = (L.off_words + n_groups * 4 + 255) / 256 * 256;
+	L.off_sums = (L.off_cuts + n_groups * 8 + 255) / 256 * 256;
 	L.off_items = (L.off_sums + (n_groups / PREPARE_WAVES + 1) * 4 + 255) / 256 * 256;
 	L.off_list = (L.off_items + n_items * 8 + 255) / 256 * 256;
 	L.off_side = (L.off_list + n_groups * 4 + 255) / 256 * 256;
 	L.bytes = L.off_side + n_groups * fused::RAYS * 4;
 	return L;
 }
-static ChainScratch chain_scratch_at(void* base, uint32_t n_rays, uint32_t* host_error, uint32_t spin_limit) {
-	const ChainLayout L = chain_layout(n_rays);
+static ChainScratch chain_scratch_at(void* base, uint32_t n_rays, uint32_t max_parts, uint32_t* host_error, uint32_t spin_limit) {
+	const ChainLayout L = chain_layout(n_rays, max_parts);
 	ChainScratch S;
 	S.item_status = (unsigned long long*)base;
 	S.seg_status = (unsigned long long*)((char*)base + L.off_seg);
@@ -72,14 +74,20 @@ static ChainScratch chain_scratch_at(void* base, uint32_t n_rays, uint32_t* host
 	S.slow_count = S.initial + 2;
 	S.n_items = S.initial + 3;
 	S.group_words = (uint32_t*)((char*)base + L.off_words);
+	S.group_cuts = (unsigned long long*)((char*)base + L.off_cuts);
 	S.prepare_sums = (uint32_t*)((char*)base + L.off_sums);
 	S.items = (U2*)((char*)base + L.off_items);
 	S.slow_items = (uint32_t*)((char*)base + L.off_list);
 	S.side = (uint32_t*)((char*)base + L.off_side);
 	S.host_error = host_error;
 	S.spin_limit = spin_limit;
+	S.max_parts = max_parts;
 	return S;
 }
+// Items a group may be cut into: any number where the scratch is allocated to fit; the scratch that is part of the library's
+// image (see g_noalloc_scratch) has room for eight, and groups that need more take the path of the listed ones there.
+constexpr uint32_t STREAM_MAX_PARTS = fused::MAX_PARTS;
+constexpr uint32_t NOALLOC_MAX_PARTS = 8;
 
 // Ordering point between the phases of a group (see srf_composite_fused.h): a workgroup barrier.
 __device__ __forceinline__ void group_sync() { __syncthreads(); }
@@ -87,13 +95,13 @@ __device__ __forceinline__ void group_sync() { __syncthreads(); }
 // ---- groups that do not fit the streaming path ------------------------------------------------
 // The streaming kernel takes groups whose rays are laid out back to back and whose samples fit one of its windows.  The
 // others (arbitrary caller-supplied offsets; more samples than one window) are rare and are kept out of its code:
-//   k_chain_prepare      clears the chain's status words, plans every group and notes how many items it makes
-//   k_chain_items        numbers the items in ray order and lists those of groups that the streaming path does not take
+//   k_chain_prepare      plans every group and notes how many items it makes
+//   k_chain_items        numbers the items in ray order, clears their words of the chain and lists those of groups that the streaming path does not take
 //   k_slow_groups (fwd)  forward pass of the listed groups; leaves the number of samples every one of their rays consumes
 //   k_composite_stream   for a listed group only chains those counts to its neighbours' and leaves the rays' compacted offsets
 //   k_slow_groups (bwd)  forward pass again, then commit and gradients at those offsets
-// Rays not laid out back to back are composited one lane per ray; groups longer than a window run the window phases over
-// all windows.
+// Rays not laid out back to back are composited one lane per ray; groups with a ray longer than a window run the window
+// phases over all windows.
 
 // Records of one group into a plan, by the 64 lanes of one wave: what fused::plan_lane and fused::plan_finish_lane
 // compute lane by lane through LDS, with the wave's own reductions instead (64 lanes adding to one LDS word take turns).
@@ -131,8 +139,29 @@ __device__ __forceinline__ U2 load_record(uint32_t g, uint32_t lane, const fused
 	return rec;
 }
 
+// fused::plan_cuts by the 64 lanes of the wave that wrote the plan: lane r holds where ray r begins and ends, one ballot finds
+// the first ray that does not fit with the rays from `lo` on (the ends only grow), so a group costs one round per item.
+__device__ __forceinline__ uint64_t plan_cuts_wave(uint32_t lane, const fused::Plan& pl, uint32_t win, uint32_t max_parts) {
+	using namespace fused;
+	if (pl.misc[M_CONTIG] == 0) return 0ull;
+	if (pl.misc[M_TOTAL] <= win) return 1ull;
+	const uint32_t start = pl.rbase[lane], end = pl.rbase[lane + 1];      // rbase[RAYS]: the group's end
+	uint64_t cuts = 1ull;
+	uint32_t parts = 1, lo = 0;
+	for (;;) {
+		const uint32_t lo_base = lane_value_u32(start, lo);
+		const uint64_t beyond = __ballot(end - lo_base > win) & ~((1ull << lo) - 1ull);
+		if (beyond == 0ull) return cuts;
+		const uint32_t r = (uint32_t)__builtin_ctzll(beyond);
+		if (r == lo) return 0ull;                      // ray lo alone does not fit
+		lo = r;
+		cuts |= 1ull << lo;
+		if (++parts > max_parts) return 0ull;
+	}
+}
+
 // One wave per group, PREPARE_WAVES groups per workgroup; a workgroup also leaves the number of items its groups make.
-__global__ void __launch_bounds__(PREPARE_WAVES * WAVE) k_chain_prepare(fused::Args A, const uint32_t* __restrict__ n_rays_counter, ChainScratch S, uint32_t n_groups_max,
+__global__ void __launch_bounds__(PREPARE_WAVES * WAVE) k_chain_prepare(fused::Args A, const uint32_t* __restrict__ n_rays_counter, ChainScratch S,
                                                                        const uint32_t* __restrict__ counter) {
 	using namespace fused;
 	__shared__ Plan plans[PREPARE_WAVES];
@@ -140,18 +169,18 @@ __global__ void __launch_bounds__(PREPARE_WAVES * WAVE) k_chain_prepare(fused::A
 	const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
 	const uint32_t g = blockIdx.x * PREPARE_WAVES + wave;
 	if (blockIdx.x == 0 && threadIdx.x == 0) { *S.initial = *counter; *S.error = 0u; *S.slow_count = 0u; }
-	if (g < n_groups_max) {
-		if (lane < 2) S.item_status[2 * g + lane] = 0ull;
-		if (lane == 0 && g % 32 == 0) { S.seg_status[(size_t)(g / 32) * SEG_STRIDE] = 0ull; S.seg_prefix[g / 32] = 0ull; }
-	}
 	const uint32_t counter_now = *n_rays_counter;
 	A.n_active = counter_now < A.K.n_rays ? counter_now : A.K.n_rays;
 	uint32_t word = 0;
 	if (g < div_up(A.n_active, RAYS)) {
 		Plan& pl = plans[wave];
 		plan_from_records(lane, g, load_record(g, lane, A), A, pl);
-		word = group_items_word<StreamGeometry>(pl);
-		if (lane == 0) S.group_words[g] = word;
+		const uint64_t cuts = plan_cuts_wave(lane, pl, StreamGeometry::WIN, S.max_parts);
+		word = group_items_word(cuts);
+		if (lane == 0) {
+			S.group_words[g] = word;
+			if ((word & 0xffu) > 1u) S.group_cuts[g] = cuts;
+		}
 	}
 	if (lane == 0) n_items_of_wave[wave] = word & 0xffu;
 	__syncthreads();
@@ -187,11 +216,13 @@ __global__ void __launch_bounds__(ITEMS_THREADS) k_chain_items(uint32_t n_rays_m
 	for (uint32_t k = 0; k < ITEMS_THREADS / WAVE; ++k) { const uint32_t t = wave_total[k]; base += wave_before[k] + (k < wave ? t : 0u); all += wave_before[k] + t; }
 	if (n != 0) {
 		const uint32_t first = base + incl - n;
-		U2 it[2];
-		items_of_group(g, word, it);
-		S.items[first] = it[0];
-		if (n == 2) S.items[first + 1] = it[1];
-		if (item_listed(it[0])) S.slow_items[atomicAdd(S.slow_count, 1u)] = first;
+		items_of_group(g, word, n > 1u ? S.group_cuts[g] : 1ull, S.items + first);
+		if ((word & (1u << 16)) != 0u) S.slow_items[atomicAdd(S.slow_count, 1u)] = first;
+		// the chain's words of these items, and of the segments of 64 items that begin with one of them
+		for (uint32_t i = first; i < first + n; ++i) {
+			S.item_status[i] = 0ull;
+			if (i % WAVE == 0) { S.seg_status[(size_t)(i / WAVE) * SEG_STRIDE] = 0ull; S.seg_prefix[i / WAVE] = 0ull; }
+		}
 	}
 	if (tid == 0 && g_first + ITEMS_THREADS >= n_groups) *S.n_items = all;     // the workgroup with the last group
 }
@@ -675,7 +706,7 @@ static int launch_stream(const srf_loss_args* a, const LossConst& K, ChainScratc
 #undef SRF_RESIDENT
 	if (rc != SRF_OK) return rc;
 	const dim3 grid(n_groups < resident ? n_groups : resident), block(STREAM_THREADS), slow_block(fused::WideGeometry::THREADS), slow_grid(n_groups < 256u ? n_groups : 256u);   // listed groups are few
-	hipLaunchKernelGGL(k_chain_prepare, dim3(div_up(n_groups, PREPARE_WAVES)), dim3(PREPARE_WAVES * WAVE), 0, st, A, n_rays_counter, S, n_groups, (const uint32_t*)n_compacted_coords_counter);
+	hipLaunchKernelGGL(k_chain_prepare, dim3(div_up(n_groups, PREPARE_WAVES)), dim3(PREPARE_WAVES * WAVE), 0, st, A, n_rays_counter, S, (const uint32_t*)n_compacted_coords_counter);
 	hipLaunchKernelGGL(k_chain_items, dim3(div_up(n_groups, ITEMS_THREADS)), dim3(ITEMS_THREADS), 0, st, a->n_rays, n_rays_counter, S);
 	SRF_LAUNCH_CHECK();
 	if (hin) hipLaunchKernelGGL((k_slow_groups<true, false, false>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S);
@@ -823,7 +854,7 @@ static int loss_call_prepare(srf_marcher* m, const srf_loss_args* a, const float
 // The chain's scratch for srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: part of the library's image on every
 // device, found once per device with hipGetSymbolAddress (the array's name means nothing to host code).
 constexpr uint32_t NOALLOC_MAX_RAYS = SRF_NOALLOC_MAX_RAYS;
-constexpr size_t NOALLOC_BYTES = chain_layout(NOALLOC_MAX_RAYS).bytes;
+constexpr size_t NOALLOC_BYTES = chain_layout(NOALLOC_MAX_RAYS, NOALLOC_MAX_PARTS).bytes;
 static __device__ __align__(256) unsigned char g_noalloc_scratch[NOALLOC_BYTES];
 constexpr int NOALLOC_MAX_DEVICES = 64;
 static void* g_noalloc_ptr[NOALLOC_MAX_DEVICES];      // per device: where g_noalloc_scratch lies in its memory
@@ -942,10 +973,10 @@ int srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const 
 		                    compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, st);
 	}
 	if (fusable && level == 0) {
-		rc = m->ws.reserve(chain_layout(a->n_rays).bytes);
+		rc = m->ws.reserve(chain_layout(a->n_rays, STREAM_MAX_PARTS).bytes);
 		if (rc != SRF_OK) return rc;
-		m->chain_error_dev = chain_scratch_at(m->ws.ptr, a->n_rays, nullptr, 0).error;
-		return launch_stream(a, K, chain_scratch_at(m->ws.ptr, a->n_rays, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
+		m->chain_error_dev = chain_scratch_at(m->ws.ptr, a->n_rays, STREAM_MAX_PARTS, nullptr, 0).error;
+		return launch_stream(a, K, chain_scratch_at(m->ws.ptr, a->n_rays, STREAM_MAX_PARTS, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
 		                     compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, st);
 	}
 
@@ -1002,8 +1033,8 @@ int srf_marcher_volume_rendering_with_loss_and_gradient_noalloc(srf_marcher_t* m
 	void* scratch = nullptr;
 	rc = noalloc_scratch(&scratch);
 	if (rc != SRF_OK) return rc;
-	m->chain_error_dev = chain_scratch_at(scratch, a->n_rays, nullptr, 0).error;
-	return launch_stream(a, K, chain_scratch_at(scratch, a->n_rays, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
+	m->chain_error_dev = chain_scratch_at(scratch, a->n_rays, NOALLOC_MAX_PARTS, nullptr, 0).error;
+	return launch_stream(a, K, chain_scratch_at(scratch, a->n_rays, NOALLOC_MAX_PARTS, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
 	                     compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, (hipStream_t)stream);
 }
 

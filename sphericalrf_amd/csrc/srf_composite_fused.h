@@ -97,20 +97,27 @@ struct Plan {
 template <class G>
 SRF_HD bool plan_fits_one_window(const Plan& pl) { return pl.misc[M_CONTIG] != 0 && pl.misc[M_TOTAL] <= G::WIN; }
 
-// In how many parts a kernel with windows of G::WIN samples takes a planned group: 1 when it fits one window, 2 when
-// it can be cut at a ray boundary into two stretches that each fit one (rays [0, *split) and [*split, RAYS)), 0 when
-// it cannot (rays not laid out back to back, a single ray longer than a window, more than two windows' worth).
+// Where a kernel with windows of G::WIN samples cuts a planned group into items: bit r of the result is set when an item
+// starts at ray r.  Greedy from the front: an item takes rays for as long as the stretch from its first ray's first sample to
+// the next ray's first sample (the group's end after the last ray) fits one window.  0 when the kernel cannot take the group:
+// rays not laid out back to back, a single ray longer than a window, more than max_parts items.
+constexpr uint32_t MAX_PARTS = RAYS;     // at worst every ray is an item of its own
 template <class G>
-SRF_HD uint32_t plan_parts(const Plan& pl, uint32_t* split) {
-	*split = RAYS;
-	if (pl.misc[M_CONTIG] == 0) return 0;
+SRF_HD uint64_t plan_cuts(const Plan& pl, uint32_t max_parts) {
+	if (pl.misc[M_CONTIG] == 0) return 0ull;
 	const uint32_t total = pl.misc[M_TOTAL];
-	if (total <= G::WIN) return 1;
-	uint32_t s = 0;                                   // the last ray that starts inside the first window
-	for (uint32_t r = 1; r < RAYS; ++r) if (pl.rbase[r] <= G::WIN) s = r;
-	if (s == 0 || total - pl.rbase[s] > G::WIN) return 0;
-	*split = s;
-	return 2;
+	if (total <= G::WIN) return 1ull;
+	uint64_t cuts = 1ull;
+	uint32_t parts = 1, lo = 0;
+	for (uint32_t r = 1; r <= RAYS; ++r) {
+		const uint32_t end = r < RAYS ? pl.rbase[r] : total;      // where ray r - 1 and the gap after it end
+		if (end - pl.rbase[lo] <= G::WIN) continue;
+		if (r - 1 == lo) return 0ull;                              // ray lo alone does not fit
+		lo = r - 1;
+		cuts |= 1ull << lo;
+		if (++parts > max_parts || end - pl.rbase[lo] > G::WIN) return 0ull;
+	}
+	return cuts;
 }
 
 // The plan of rays [lo, hi) of a planned group, one lane per ray: the other rays own nothing in it.
@@ -134,22 +141,29 @@ SRF_HD void plan_part_lane(uint32_t lane, const Plan& group, uint32_t lo, uint32
 	}
 }
 
-// An item is what a streaming workgroup takes at a time: rays [lo, hi) of one group.  A group is one item, or two when
-// it is cut (plan_parts), and the items of all groups, in ray order, are the units of the ordered-offset chain.
+// An item is what a streaming workgroup takes at a time: rays [lo, hi) of one group.  A group is one item, or several when
+// it is cut (plan_cuts), and the items of all groups, in ray order, are the units of the ordered-offset chain.
 //   x  group
-//   y  lo | hi << 8 | listed << 16   (listed: the streaming path does not take the group, see plan_parts == 0)
-// What k_chain_prepare leaves per group for the pass that numbers the items: items | split << 8 | listed << 16.
-template <class G>
-SRF_HD uint32_t group_items_word(const Plan& pl) {
-	uint32_t split;
-	const uint32_t parts = plan_parts<G>(pl, &split);
-	return (parts == 2 ? 2u : 1u) | (split << 8) | (parts == 0 ? 1u << 16 : 0u);
+//   y  lo | hi << 8 | listed << 16   (listed: the streaming path does not take the group, see plan_cuts == 0)
+// What k_chain_prepare leaves per group for the pass that numbers the items: items | listed << 16 (and the cuts themselves
+// when there are several).
+SRF_HD uint32_t group_items_word(uint64_t cuts) { return cuts ? (uint32_t)__builtin_popcountll(cuts) : (1u | 1u << 16); }
+SRF_HD U2 make_item(uint32_t g, uint32_t lo, uint32_t hi, bool listed) {
+	U2 item;
+	item.x = g;
+	item.y = lo | (hi << 8) | (listed ? 1u << 16 : 0u);
+	return item;
 }
-SRF_HD uint32_t items_of_group(uint32_t g, uint32_t word, U2 out[2]) {
-	const uint32_t n = word & 0xffu, split = (word >> 8) & 0xffu, listed = word & (1u << 16);
-	out[0].x = g; out[1].x = g;
-	if (n == 2) { out[0].y = 0u | (split << 8); out[1].y = split | (RAYS << 8); }
-	else { out[0].y = (RAYS << 8) | listed; out[1].y = 0; }
+// the items of a group in ray order, written to out[0 .. n): the whole group when it is listed or not cut
+SRF_HD uint32_t items_of_group(uint32_t g, uint32_t word, uint64_t cuts, U2* out) {
+	const uint32_t n = word & 0xffu;
+	const bool listed = (word & (1u << 16)) != 0u;
+	if (listed || n <= 1u) { out[0] = make_item(g, 0u, RAYS, listed); return 1u; }
+	for (uint32_t k = 0; k < n; ++k) {
+		const uint32_t lo = (uint32_t)__builtin_ctzll(cuts);
+		cuts &= cuts - 1ull;
+		out[k] = make_item(g, lo, cuts ? (uint32_t)__builtin_ctzll(cuts) : RAYS, false);
+	}
 	return n;
 }
 SRF_HD uint32_t item_lo(U2 item) { return item.y & 0xffu; }

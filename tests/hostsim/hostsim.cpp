@@ -55,6 +55,9 @@ static LossConst make_loss_const(const orc_loss_args* a) {
 // forward pass first and leave their per-ray counts; the streaming loop then runs every group in order (count, chain
 // with the count known, finish, ordered offsets, phase C), handing the listed groups only their offsets; the listed
 // groups' second forward pass and their gradients come last.
+// items a group may be cut into (what the device's scratch has room for), and the most that a group of the last call made
+static uint32_t g_fused_max_parts = fused::MAX_PARTS, g_fused_most_parts = 0;
+
 template <bool HI, bool HO>
 static void run_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n_rays_counter, uint32_t* ray_coord_indices, const float* dt,
                       const float* coords, float* compacted_coords, uint32_t* n_compacted_counter, const void* net, void* dloss, float* loss_output,
@@ -91,9 +94,11 @@ static void run_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n
 	std::vector<U2> items;
 	for (uint32_t g = 0; g < n_groups; ++g) {
 		make_plan(g, plans[0], nullptr);
-		const uint32_t word = group_items_word<GS>(plans[0]);
-		U2 it[2];
-		const uint32_t n = items_of_group(g, word, it);
+		const uint64_t cuts = plan_cuts<GS>(plans[0], g_fused_max_parts);
+		const uint32_t word = group_items_word(cuts);
+		U2 it[MAX_PARTS];
+		const uint32_t n = items_of_group(g, word, cuts, it);
+		g_fused_most_parts = n > g_fused_most_parts ? n : g_fused_most_parts;
 		if (item_listed(it[0])) {
 			slow.push_back(g);
 			if (plans[0].misc[M_CONTIG] == 0) ++*n_scattered_groups; else ++*n_multi_window_groups;
@@ -732,11 +737,15 @@ void hs_loss(const orc_loss_args* a, const float* rays_rgba, uint32_t n_rays_cou
 	}
 }
 
+void hs_fused_set_max_parts(uint32_t n) { g_fused_max_parts = n; }
+uint32_t hs_fused_most_parts() { return g_fused_most_parts; }
+
 void hs_loss_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n_rays_counter, uint32_t* ray_coord_indices, const float* dt,
                    const float* coords, float* compacted_coords, uint32_t* n_compacted_counter, const void* net, void* dloss, float* loss_output,
                    float* rgb_ray_out, uint32_t* n_scattered_groups, uint32_t* n_multi_window_groups) {
 	const bool hin = a->network_output_dtype == ORC_DTYPE_F16, hout = a->dloss_dtype == ORC_DTYPE_F16;
 	*n_scattered_groups = 0; *n_multi_window_groups = 0;
+	g_fused_most_parts = 0;
 #define RUN(HI, HO) run_fused<HI, HO>(a, rays_rgba, n_rays_counter, ray_coord_indices, dt, coords, compacted_coords, n_compacted_counter, net, dloss, loss_output, rgb_ray_out, n_scattered_groups, n_multi_window_groups)
 	if (hin && hout) RUN(true, true); else if (hin) RUN(true, false); else if (hout) RUN(false, true); else RUN(false, false);
 #undef RUN

@@ -22,6 +22,10 @@ def layout(rng, kind, n_rays):
     elif kind == "split":        # groups longer than one window of the streaming kernel, cut at a ray boundary into two parts
         counts = rng.integers(25, 60, n_rays)
         counts[n_rays // 3:n_rays // 3 + 40] = rng.integers(0, 12, 40)
+    elif kind == "parts":        # groups of many windows' worth of samples, none of whose rays exceeds a window: cut into several parts
+        counts = rng.integers(60, 400, n_rays)
+        counts[70:90] = rng.integers(1000, 1900, 20)
+        counts[130:150] = 0
     elif kind == "tiny":
         counts = rng.integers(0, 3, n_rays)
     else:
@@ -40,14 +44,14 @@ def layout(rng, kind, n_rays):
     return counts.astype(np.uint32), base.astype(np.uint32), total
 
 
-@pytest.mark.parametrize("kind", ["short", "long", "split", "tiny", "gaps", "biggap", "shuffled"])
+@pytest.mark.parametrize("kind", ["short", "long", "split", "parts", "tiny", "gaps", "biggap", "shuffled"])
 @pytest.mark.parametrize("hin,hout", [(False, False), (True, False), (True, True)])
 def test_fused_equals_oracle(orc, hostsim, kind, hin, hout):
-    rng = np.random.default_rng(["short", "long", "tiny", "gaps", "biggap", "shuffled", "split"].index(kind) + 100)
+    rng = np.random.default_rng(["short", "long", "tiny", "gaps", "biggap", "shuffled", "split", "parts"].index(kind) + 100)
     n_rays = 64 * 5 + 17
     counts, base, total = layout(rng, kind, n_rays)
     net = helpers.random_network_output(rng, total, np.float16 if hin else np.float32)
-    net[:, 3] *= (0.05 if kind == "long" else 3)
+    net[:, 3] *= (0.05 if kind in ("long", "parts") else 3)
     coords = rng.random((total, 7)).astype(np.float32)
     coords[:, 3] = coords[:, 3] * 0.3 + 0.01
     tgt = rng.random((n_rays, 4)).astype(np.float32)
@@ -57,7 +61,7 @@ def test_fused_equals_oracle(orc, hostsim, kind, hin, hout):
               background_color=(O.f32 * 3)(0.1, 0.7, 0.3), mean_density=0.001)
     a = loss_args(n_rays, cap, **kw)
     outs = []
-    for fn in ("oracle", "fused", "wave", "wave_stride_128", "wave_stride_4096"):
+    for fn in ("oracle", "fused", "fused_8_parts", "wave", "wave_stride_128", "wave_stride_4096"):
         idx = np.stack([counts, base], axis=1).astype(np.uint32)
         dloss = np.zeros((cap, 4), np.float16 if hout else np.float32)
         comp = np.zeros((cap, 7), np.float32)
@@ -81,24 +85,34 @@ def test_fused_equals_oracle(orc, hostsim, kind, hin, hout):
             if kind == "shuffled" or table_overflows:
                 assert in_window == 0 and chunked == 0 and per_ray == (n_active + 63) // 64
             else:
-                assert per_ray == 0 and in_window > 0
-                if kind == "long":
+                assert per_ray == 0 and (in_window > 0 or kind == "parts")
+                if kind in ("long", "parts"):
                     assert chunked > 0
-                if stride == 4096:
+                if stride == 4096 and kind != "parts":
                     assert several > 0      # more than 64 rays start in windows of that size
                 if stride == 0 and kind in ("short", "split", "gaps"):
                     assert several == 0 and chunked == 0
         else:
+            # the streaming kernel's control flow, with groups cut into as many items as it takes, and into eight at most (the
+            # limit of the entry point that allocates nothing: groups that need more take the path of the listed ones)
             cnt = np.array([11], np.uint32)
             ns, nm = C.c_uint32(), C.c_uint32()
+            hostsim.lib.hs_fused_set_max_parts(8 if fn == "fused_8_parts" else 64)
             hostsim.lib.hs_loss_fused(C.byref(a), ptr(tgt), n_active, ptr(idx), ptr(dt), ptr(coords), ptr(comp), ptr(cnt), ptr(net), ptr(dloss),
                                       ptr(loss), ptr(rgb), C.byref(ns), C.byref(nm))
+            hostsim.lib.hs_fused_set_max_parts(64)
+            hostsim.lib.hs_fused_most_parts.restype = C.c_uint32
+            most = hostsim.lib.hs_fused_most_parts()
             tot = int(cnt[0])
             if kind in ("shuffled", "biggap"):
                 assert ns.value > 0
             else:
                 assert ns.value == 0
-            assert (nm.value > 0) == (kind == "long")
+            assert (nm.value > 0) == (kind == "long" or (kind == "parts" and fn == "fused_8_parts"))
+            if kind == "split":
+                assert most == 2
+            if kind == "parts":
+                assert most > 8 if fn == "fused" else 2 < most <= 8
         outs.append((tot, idx, dloss.view(np.uint16 if hout else np.uint32), comp, loss, rgb))
     for other in outs[1:]:
         for name, x, y in zip(("total", "idx", "dloss", "compacted_coords", "loss", "rgb"), outs[0], other):

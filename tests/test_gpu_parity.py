@@ -1101,10 +1101,10 @@ def test_errors_are_reported_not_thrown_across_the_abi(gpu):
 
 @pytest.mark.parametrize("impl", ["waves", "stream"])
 @pytest.mark.parametrize("acts", ["plain", "activated", "relu"])
-@pytest.mark.parametrize("kind", ["short", "long", "split", "tiny", "gaps", "biggap", "shuffled"])
+@pytest.mark.parametrize("kind", ["short", "long", "split", "parts", "tiny", "gaps", "biggap", "shuffled"])
 def test_single_launch_compositing_layouts(gpu, orc, kind, acts, impl, monkeypatch):
-    """every sample layout the streaming compositing distinguishes (back-to-back rays, holes, groups longer than a window,
-    shuffled offsets), against the oracle, over many workgroups so that its ordered offsets really go through the chain;
+    """every sample layout the streaming compositing distinguishes (back-to-back rays, holes, groups longer than a window cut
+    into two or into many items, rays longer than a window, shuffled offsets), against the oracle, over many workgroups so that its ordered offsets really go through the chain;
     with the activations compiled out ("plain": both None) and with the run-time switches (Logistic colour and Exponential density;
     ReLU for both, over outputs of either sign)"""
     monkeypatch.setenv("SRF_COMPOSITE_IMPL", impl)
@@ -1112,16 +1112,16 @@ def test_single_launch_compositing_layouts(gpu, orc, kind, acts, impl, monkeypat
     torch = gpu
     from sphericalrf_amd import api
     from tests.test_fused_compositing_on_host import layout
-    rng = np.random.default_rng(["short", "long", "tiny", "gaps", "biggap", "shuffled", "split"].index(kind) + 200)
-    n_rays = 64 * 700 + 29
+    rng = np.random.default_rng(["short", "long", "tiny", "gaps", "biggap", "shuffled", "split", "parts"].index(kind) + 200)
+    n_rays = 64 * (150 if kind == "parts" else 700) + 29
     counts, base, total = layout(rng, kind, n_rays)
     net = helpers.random_network_output(rng, total, np.float16)
-    net[:, 3] *= np.float16(0.05 if kind == "long" else 3)
+    net[:, 3] *= np.float16(0.05 if kind in ("long", "parts") else 3)
     if acts == "activated":
         net[:, 3] = np.log(net[:, 3].astype(np.float32) + 1e-3).astype(np.float16)      # the exponential brings the densities back
     if acts == "relu":
         net[:, :3] -= np.float16(0.3)          # a third of the colours and of the densities below zero: clamped, with zero derivative
-        net[:, 3] -= np.float16(0.4 * (0.05 if kind == "long" else 3))
+        net[:, 3] -= np.float16(0.4 * (0.05 if kind in ("long", "parts") else 3))
     dt = (rng.random(total) * 0.3 + 0.01).astype(np.float32)
     tgt = rng.random((n_rays, 4)).astype(np.float32)
     cap = int(counts.sum() * 0.9) + 1

@@ -54,7 +54,8 @@ def test_no_alloc_entry_point_matches_the_ordinary_one_twice_in_a_row(gpu, monke
     ordinary, no_alloc = api.RayMarcher(cfg), api.RayMarcher(cfg)
     first = _inputs(torch, 41, 64 * 900 + 17, "gaps")      # several segments of items, holes between rays
     second = _inputs(torch, 42, 64 * 40 + 5, "split")      # smaller, with groups that are cut into two items
-    for w in (first, second):
+    third = _inputs(torch, 45, 64 * 30 + 7, "parts")       # groups of many windows: cut into items by one entry point, beyond the other's limit of eight
+    for w in (first, second, third):
         want = _run(torch, api, ordinary, w, False)
         got = _run(torch, api, no_alloc, w, True)
         assert int(want[0][0]) > 5
