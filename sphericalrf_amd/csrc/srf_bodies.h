@@ -287,8 +287,9 @@ struct CountArgs {
 	uint32_t* counts;
 	StepLog log;
 	SkipTable skip;
-	// parking: budget of probes per ray (0 = never park), the queue, its capacity, its fill counter
-	uint32_t probe_budget;
+	// parking: budget of probes per ray (0 = never park), the queue, its capacity, its fill counter; a wavefront only parks
+	// rays once it has no more than park_lanes rays under way
+	uint32_t probe_budget, park_lanes;
 	ParkedRay* parked;
 	uint32_t parked_capacity;
 	uint32_t* parked_count;
@@ -434,7 +435,7 @@ SRF_HD void count_unpark(CountLane& L, const ParkedRay& r) {
 // occupancy_sampler.cu:595-628 — a step that looks its cell up
 // SPHERE = false compiles the optional sphere bound out (the counting kernel is short of registers; it is built both ways)
 template <bool SPHERE = true>
-SRF_HD void count_probe(CountLane& L, const Params& P, const CountArgs& A) {
+SRF_HD void count_probe(CountLane& L, const Params& P, const CountArgs& A, bool may_park = true) {
 	const Vec3 pos = along(L.o, L.d, L.t);
 	if (!(aabb_contains(P, pos) && L.j < P.n_max_steps)) { count_finish(L, A); return; }
 	if (SPHERE && P.sphere[3] > 0.f) {      // optional sphere bound: no sample outside it, the chain of t as it is
@@ -448,7 +449,7 @@ SRF_HD void count_probe(CountLane& L, const Params& P, const CountArgs& A) {
 			return;
 		}
 	}
-	if (A.probe_budget && L.probes >= A.probe_budget && count_park(L, A)) return;
+	if (may_park && A.probe_budget && L.probes >= A.probe_budget && count_park(L, A)) return;
 	++L.probes;
 	SRF_COUNT_PROBE();
 	const Probe s = probe_at(P, P.use_grid ? A.bitfield : nullptr, pos, L.t, P.cone_angle_constant, &A.skip);

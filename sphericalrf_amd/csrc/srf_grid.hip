@@ -716,6 +716,8 @@ int srf_sampler_create(const srf_sampler_config* c, srf_sampler_t** out) {
 	s->force_sample_by_cell = tri_state("SRF_GRID_SAMPLE_BY_CELL");
 	s->count_probe_budget = COUNT_PROBE_BUDGET;
 	{ const char* v = getenv("SRF_COUNT_PROBE_BUDGET"); if (v && v[0]) s->count_probe_budget = (uint32_t)atoi(v); }
+	s->count_park_lanes = COUNT_PARK_LANES;
+	{ const char* v = getenv("SRF_COUNT_PARK_LANES"); if (v && v[0]) s->count_park_lanes = (uint32_t)atoi(v); }
 	// SRF_MARCH_PARK_ALL=1: the render marches hand every ray that finds an empty cell without anything to skip to their
 	// one-ray-per-wavefront march at once, whatever the wavefront still holds (for tests: that march then does most of a frame)
 	{ const char* v = getenv("SRF_MARCH_PARK_ALL"); s->march_park_all = v && v[0] == '1'; }

@@ -28,6 +28,7 @@ struct Workspace {
 };
 
 constexpr uint32_t COUNT_PROBE_BUDGET = 192;   // lookups after which the counting march parks a ray for the wide march
+constexpr uint32_t COUNT_PARK_LANES = 32;      // ... once its wavefront has no more rays than this under way
 
 SRF_HD uint32_t div_up(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 inline size_t align_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
@@ -58,9 +59,10 @@ struct srf_sampler {
 	// Switches the tests use to run both sides of a size-dependent choice on small inputs; read from the environment once, when the
 	// sampler is created (-1: the library chooses): SRF_SPLAT_SORT, SRF_GRID_SAMPLE_BITS, SRF_GRID_SAMPLE_BY_CELL = 0|1
 	// (SRF_SPLAT_SORT=2: the large-batch splat through the library's radix sort instead of the partition made for it);
-	// SRF_COUNT_PROBE_BUDGET = lookups after which the counting march parks a ray (0: never)
+	// SRF_COUNT_PROBE_BUDGET = lookups after which the counting march parks a ray (0: never), SRF_COUNT_PARK_LANES = rays a
+	// wavefront may have under way when it does
 	int      force_splat_sort, force_sample_bits, force_sample_by_cell;
-	uint32_t count_probe_budget;
+	uint32_t count_probe_budget, count_park_lanes;
 	bool     grid_sample_cell_order = false;   // srf_sampler_set_grid_sample_order
 	uint32_t dealt_entries = 0;                // leading entries the last sample_positions_from_grid left in cell order
 	srf::Workspace ws;

@@ -84,7 +84,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(SRF_COU
 			if (L.phase == LANE_STEP) count_steps<COUNT_STEP_BURST>(L, P, A);
 			SRF_COUNT_STAMP(0, n_step);
 		} else if (!begin) {
-			if (L.phase == LANE_PROBE) count_probe<SPHERE>(L, P, A);
+			if (L.phase == LANE_PROBE) count_probe<SPHERE>(L, P, A, n_probe + n_step <= A.park_lanes);
 			SRF_COUNT_STAMP(1, n_probe);
 		} else {
 			const uint32_t rank = (uint32_t)__popcll(m_idle & ((1ull << lane) - 1ull));
@@ -607,6 +607,7 @@ int srf_sampler_sample_coords_from_dataset(srf_sampler_t* s, uint32_t n_rays, ui
 	ca.state = state; ca.counts = counts; ca.log = log;
 	ca.skip = sampler_skip_table(s);
 	ca.probe_budget = probe_budget;
+	ca.park_lanes = s->count_park_lanes;
 	ca.parked = (ParkedRay*)(w + off_parked);
 	ca.parked_capacity = parked_capacity;
 	ca.parked_count = (uint32_t*)(w + off_parked_count);

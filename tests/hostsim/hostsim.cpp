@@ -488,7 +488,7 @@ void hs_generate_training_samples(const orc_params* p, uint32_t n_rays, uint32_t
 	// a queue smaller than the number of rays exercises the refusal as well
 	std::vector<ParkedRay> parked(probe_budget ? n_rays / 2 + 1 : 0);
 	uint32_t parked_count = 0;
-	ca.probe_budget = probe_budget; ca.parked = parked.data(); ca.parked_capacity = (uint32_t)parked.size(); ca.parked_count = &parked_count;
+	ca.probe_budget = probe_budget; ca.park_lanes = 64; ca.parked = parked.data(); ca.parked_capacity = (uint32_t)parked.size(); ca.parked_count = &parked_count;
 	// rays_per_wave 0: every ray start to end on its own; otherwise wavefronts of 64 lanes sharing rays_per_wave rays as on the device
 	if (rays_per_wave == 0) for (uint32_t i = 0; i < n_rays; ++i) train_count_body(i, P, ca);
 	else {

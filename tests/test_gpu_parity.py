@@ -240,6 +240,7 @@ def test_training_sampler(gpu, orc, config_id, scale, budget, monkeypatch):
     torch = gpu
     if budget is not None:
         monkeypatch.setenv("SRF_COUNT_PROBE_BUDGET", budget)
+        monkeypatch.setenv("SRF_COUNT_PARK_LANES", "64")      # park whatever else the wavefront has under way
     from sphericalrf_amd import api
     w, p, grid, bf, mean = helpers.build_scene(orc, config_id, scale)
     s = make_sampler(torch, api, w, grid)
@@ -525,8 +526,10 @@ def test_full_size_march_is_the_same_whatever_the_probe_budget(gpu, monkeypatch)
     for budget in (None, "0", "3", "40"):
         if budget is None:
             monkeypatch.delenv("SRF_COUNT_PROBE_BUDGET", raising=False)
+            monkeypatch.delenv("SRF_COUNT_PARK_LANES", raising=False)
         else:
             monkeypatch.setenv("SRF_COUNT_PROBE_BUDGET", budget)
+            monkeypatch.setenv("SRF_COUNT_PARK_LANES", "64" if budget == "3" else "20")      # any wavefront parks / only one down to 20 rays
         s = api.OccupancySampler(w["sampler"])      # the budget is read when a sampler is created
         s.set_density_grid(grid)
         s.update_grid_bitfield()

@@ -201,6 +201,7 @@ def test_bounded_marches_on_the_gpu(gpu, orc, hostsim, budget, monkeypatch):
     torch = gpu
     if budget is not None:
         monkeypatch.setenv("SRF_COUNT_PROBE_BUDGET", budget)      # every ray parked at its first lookup: the wide march under the bound
+        monkeypatch.setenv("SRF_COUNT_PARK_LANES", "64")
     from sphericalrf_amd import api, scene
     from tests.test_gpu_parity import make_sampler
     w, p, grid, bf, mean = helpers.build_scene(orc, 3, 1 / 8)
