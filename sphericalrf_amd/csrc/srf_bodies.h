@@ -795,11 +795,23 @@ SRF_HD void train_write_replay(uint32_t i, const Params& P, const TrainRay& st, 
 #endif
 	for (uint32_t g = 0; g < 3; ++g) {      // unrolled: the mask words stay in registers
 		uint32_t m = st.word_mask[g];
-		while (m) {
+		// a word's bits and the t at its first sample are requested while the word before it is walked
+		uint32_t next_bits = 0u;
+		float next_t = 0.f;
+		if (m) {
 			const uint32_t w = g * 32u + (uint32_t)__builtin_ctz(m);
+			next_bits = log.bits[(size_t)w * log.stride + i];
+			next_t = log.t0[(size_t)w * log.stride + i];
+		}
+		while (m) {
 			m &= m - 1u;
-			uint32_t word = log.bits[(size_t)w * log.stride + i];
-			float t = log.t0[(size_t)w * log.stride + i];   // t at the word's first sample
+			uint32_t word = next_bits;
+			float t = next_t;
+			if (m) {
+				const uint32_t w = g * 32u + (uint32_t)__builtin_ctz(m);
+				next_bits = log.bits[(size_t)w * log.stride + i];
+				next_t = log.t0[(size_t)w * log.stride + i];
+			}
 			word >>= (uint32_t)__builtin_ctz(word);
 			const bool short_form = f.usable && t >= f.t_lo;   // t only grows; the upper end is checked per step
 			ShortChain ch = short_chain_at(short_form ? t : 1.f);
