@@ -33,6 +33,7 @@ struct ChainScratch {
 	U2* items;                          // the items in ray order (fused::items_of_group)
 	uint32_t* slow_items;               // items of groups that the streaming path does not take (see k_chain_prepare)
 	uint32_t* side;                     // per ray of such a group: samples consumed (forward kernel), then compacted offset (streaming kernel)
+	U2* saved_records;                  // per ray of such a group: its record on entry, which the commit overwrites (NULL: a group is worked on by one workgroup)
 	uint32_t* host_error;               // like error, in host memory the device can write (may be NULL)
 	uint32_t spin_limit;                // polls an item makes before it gives up
 	uint32_t max_parts;                 // items a group may be cut into (what the scratch has room for)

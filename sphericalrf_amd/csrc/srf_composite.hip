@@ -45,9 +45,9 @@ __global__ void __launch_bounds__(128) k_volume_rendering(Params P, srf_render_a
 // Single-launch compositing (phases in srf_composite_fused.h)
 // ------------------------------------------------------------------------------------
 // bytes of device scratch the chain needs for n_rays rays whose groups are cut into at most max_parts items each, and where
-// its parts lie
-struct ChainLayout { size_t off_seg, off_prefix, off_misc, off_words, off_cuts, off_sums, off_items, off_list, off_side, bytes; };
-SRF_HD constexpr ChainLayout chain_layout(uint32_t n_rays, uint32_t max_parts) {
+// its parts lie (save_records: with room for a copy of the listed groups' ray records, see k_slow_groups)
+struct ChainLayout { size_t off_seg, off_prefix, off_misc, off_words, off_cuts, off_sums, off_items, off_list, off_side, off_saved, bytes; };
+SRF_HD constexpr ChainLayout chain_layout(uint32_t n_rays, uint32_t max_parts, bool save_records) {
 	const size_t n_groups = ((size_t)n_rays + fused::RAYS - 1) / fused::RAYS;
 	const size_t n_items = (size_t)max_parts * n_groups;
 	ChainLayout L = {};
@@ -60,11 +60,12 @@ SRF_HD constexpr ChainLayout chain_layout(uint32_t n_rays, uint32_t max_parts) {
 	L.off_items = (L.off_sums + (n_groups / PREPARE_WAVES + 1) * 4 + 255) / 256 * 256;
 	L.off_list = (L.off_items + n_items * 8 + 255) / 256 * 256;
 	L.off_side = (L.off_list + n_groups * 4 + 255) / 256 * 256;
-	L.bytes = L.off_side + n_groups * fused::RAYS * 4;
+	L.off_saved = (L.off_side + n_groups * fused::RAYS * 4 + 255) / 256 * 256;
+	L.bytes = L.off_saved + (save_records ? n_groups * fused::RAYS * 8 : 0);
 	return L;
 }
-static ChainScratch chain_scratch_at(void* base, uint32_t n_rays, uint32_t max_parts, uint32_t* host_error, uint32_t spin_limit) {
-	const ChainLayout L = chain_layout(n_rays, max_parts);
+static ChainScratch chain_scratch_at(void* base, uint32_t n_rays, uint32_t max_parts, bool save_records, uint32_t* host_error, uint32_t spin_limit) {
+	const ChainLayout L = chain_layout(n_rays, max_parts, save_records);
 	ChainScratch S;
 	S.item_status = (unsigned long long*)base;
 	S.seg_status = (unsigned long long*)((char*)base + L.off_seg);
@@ -79,6 +80,7 @@ static ChainScratch chain_scratch_at(void* base, uint32_t n_rays, uint32_t max_p
 	S.items = (U2*)((char*)base + L.off_items);
 	S.slow_items = (uint32_t*)((char*)base + L.off_list);
 	S.side = (uint32_t*)((char*)base + L.off_side);
+	S.saved_records = save_records ? (U2*)((char*)base + L.off_saved) : nullptr;
 	S.host_error = host_error;
 	S.spin_limit = spin_limit;
 	S.max_parts = max_parts;
@@ -105,6 +107,11 @@ __device__ __forceinline__ void group_sync() { __syncthreads(); }
 
 // Records of one group into a plan, by the 64 lanes of one wave: what fused::plan_lane and fused::plan_finish_lane
 // compute lane by lane through LDS, with the wave's own reductions instead (64 lanes adding to one LDS word take turns).
+// The streaming kernel plans an item of a cut group while the items before it may already have committed, which overwrites
+// their rays' records (count and offset after compaction).  Offsets relative to the group's first sample are therefore kept
+// modulo 2^32: in plan_part_lane the first ray's offset cancels, so a part's plan depends on the records of its own rays and
+// of the ray after them only, and that ray's item commits after this one has been planned (it waits for this one's count).
+// Whether the rays lie back to back is decided once, before anything is overwritten (k_chain_prepare), and travels with the item.
 __device__ __forceinline__ void plan_from_records(uint32_t lane, uint32_t g, U2 rec, const fused::Args& A, fused::Plan& pl) {
 	using namespace fused;
 	const uint32_t ray0 = g * RAYS;
@@ -118,9 +125,9 @@ __device__ __forceinline__ void plan_from_records(uint32_t lane, uint32_t g, U2 
 	const uint32_t sum = wave_sum_fast(mine ? rn : 0u);
 	const uint32_t last = n_here ? n_here - 1 : 0u;
 	const uint64_t end = n_here ? (uint64_t)lane_value_u32(rabs, last) + lane_value_u32(rn, last) : 0ull;
-	const uint64_t total64 = end >= s0 ? end - s0 : 0ull;
-	const uint32_t total = total64 > 0xffffffffull ? 0xffffffffu : (uint32_t)total64;
-	const bool contiguous = __ballot(out_of_order) == 0ull && !((uint64_t)total > (uint64_t)sum + GAP_SLACK);
+	const uint32_t total = (uint32_t)end - s0;
+	const bool fits = end >= s0 && end - s0 <= 0xffffffffull;
+	const bool contiguous = __ballot(out_of_order) == 0ull && fits && !((uint64_t)total > (uint64_t)sum + GAP_SLACK);
 	pl.rn[lane] = rn;
 	pl.rabs[lane] = rabs;
 	pl.rbase[lane] = mine ? rabs - s0 : total;
@@ -230,58 +237,107 @@ __global__ void __launch_bounds__(ITEMS_THREADS) k_chain_items(uint32_t n_rays_m
 struct SlowShared {
 	fused::Window<fused::WideGeometry> w;
 	fused::RayLds rl;
-	fused::Plan plan;
+	fused::Plan plan;       // the group
+	fused::Plan part;       // the rays of it that are under way
 };
 
+// Where a listed group whose rays lie back to back is cut into parts: like plan_cuts_wave, but a ray longer than a window
+// is a part of its own.  A part's rays go through the windows together and one after another part's, so that a group of long
+// rays does not walk them one behind the other; the parts of a group are dealt to `slots` units of work, which different
+// workgroups take.
+__device__ __forceinline__ uint64_t slow_cuts_wave(uint32_t lane, const fused::Plan& pl, uint32_t win) {
+	using namespace fused;
+	const uint32_t start = pl.rbase[lane], end = pl.rbase[lane + 1];
+	uint64_t cuts = 1ull;
+	uint32_t lo = 0;
+	for (;;) {
+		const uint32_t lo_base = lane_value_u32(start, lo);
+		const uint64_t beyond = __ballot(end - lo_base > win) & ~((1ull << lo) - 1ull);
+		if (beyond == 0ull) return cuts;
+		uint32_t r = (uint32_t)__builtin_ctzll(beyond);
+		if (r == lo) ++r;                              // ray lo alone is longer than a window
+		if (r >= RAYS) return cuts;
+		lo = r;
+		cuts |= 1ull << lo;
+	}
+}
+
+constexpr uint32_t SLOW_PART_SLOTS = 16;      // workgroups that share a listed group (see k_slow_groups)
+constexpr uint32_t SLOW_WORKGROUPS = 2048;
+
 template <bool HALF_IN, bool HALF_OUT, bool BACKWARD>
-__global__ void __launch_bounds__(fused::WideGeometry::THREADS) k_slow_groups(fused::Args A, const uint32_t* __restrict__ n_rays_counter, const float* __restrict__ mean_density_ptr, ChainScratch S) {
+__global__ void __launch_bounds__(fused::WideGeometry::THREADS) k_slow_groups(fused::Args A, const uint32_t* __restrict__ n_rays_counter, const float* __restrict__ mean_density_ptr, ChainScratch S, uint32_t slots) {
 	using namespace fused;
 	using G = WideGeometry;
 	__shared__ SlowShared sh;
 	const uint32_t tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
 	const uint32_t n_listed = *S.slow_count;
-	if (blockIdx.x >= n_listed) return;
+	// a unit of work: the parts of one listed group whose number is `slot` modulo `slots`
+	const uint64_t n_units = (uint64_t)n_listed * slots;
+	if (blockIdx.x >= n_units) return;
 	const uint32_t counter_now = *n_rays_counter;
 	A.mean_density = mean_density_ptr ? *mean_density_ptr : 0.f;
 	A.n_active = counter_now < A.K.n_rays ? counter_now : A.K.n_rays;
 	if (!BACKWARD) A.rgb_ray_out = nullptr;      // written once, by the second forward pass
-	Plan& pl = sh.plan;
-	for (uint32_t k = blockIdx.x; k < n_listed; k += gridDim.x) {
+	for (uint64_t unit = blockIdx.x; unit < n_units; unit += gridDim.x) {
+		const uint32_t k = (uint32_t)(unit / slots), slot = (uint32_t)(unit % slots);
 		const uint32_t g = S.items[S.slow_items[k]].x;
 		const uint32_t ray0 = g * RAYS;
-		if (wave == 0) plan_from_records(lane, g, load_record(g, lane, A), A, pl);
-		group_sync();
-		const bool live = wave == 0 && ray0 + lane < A.n_active;
-		if (pl.misc[M_CONTIG] != 0) {
-			const uint32_t n_win = (pl.misc[M_TOTAL] + G::WIN - 1) / G::WIN;
-			SlotState<G, HALF_IN> st;
-			RayCarry c;
-			Float4 target = mk4(0.f, 0.f, 0.f, 0.f);
-			if (live) target = *(const Float4*)(A.rays_rgba + 4 * (size_t)(ray0 + lane));
-			if (wave == 0) reset_carry(lane, pl, c);
-			for (uint32_t win = 0; win < n_win; ++win) {
-				phase_a<G, HALF_IN>(tid, win, A, sh.w, pl, st);
-				group_sync();
-				if (wave == 0) chain<G>(lane, win, A, sh.w, sh.rl, pl, c);
-				group_sync();
+		if (wave == 0) {
+			// The commit of the backward launch overwrites a ray's record, and the workgroups that share a group do not wait for
+			// one another: they plan from the copy that the forward launch left.
+			U2 rec;
+			if (BACKWARD && S.saved_records) rec = S.saved_records[(size_t)ray0 + lane];
+			else {
+				rec = load_record(g, lane, A);
+				if (S.saved_records && slot == 0) S.saved_records[(size_t)ray0 + lane] = rec;
 			}
-			if (wave == 0) finish_ray(lane, ray0, A, sh.rl, c, target);
-			if (!BACKWARD) {
-				if (live) S.side[ray0 + lane] = sh.rl.rnf[lane];
-			} else {
-				if (wave == 0) commit_ray(lane, ray0, live ? S.side[ray0 + lane] : 0u, A, sh.rl, pl);
+			plan_from_records(lane, g, rec, A, sh.plan);
+		}
+		group_sync();
+		if (sh.plan.misc[M_CONTIG] != 0) {
+			uint64_t cuts = slow_cuts_wave(lane, sh.plan, G::WIN);      // (the same in every wave)
+			for (uint32_t part_number = 0; cuts != 0ull; ++part_number) {
+				const uint32_t lo = (uint32_t)__builtin_ctzll(cuts);
+				cuts &= cuts - 1ull;
+				const uint32_t hi = cuts ? (uint32_t)__builtin_ctzll(cuts) : RAYS;
+				if (part_number % slots != slot) continue;
+				const Plan& pl = sh.part;
+				if (wave == 0) plan_part_lane(lane, sh.plan, lo, hi, g, sh.part);
 				group_sync();
+				const bool live = wave == 0 && ray0 + lane < A.n_active && lane >= lo && lane < hi;
+				const uint32_t n_win = (pl.misc[M_TOTAL] + G::WIN - 1) / G::WIN;
+				SlotState<G, HALF_IN> st;
+				RayCarry c;
+				Float4 target = mk4(0.f, 0.f, 0.f, 0.f);
+				if (live) target = *(const Float4*)(A.rays_rgba + 4 * (size_t)(ray0 + lane));
 				if (wave == 0) reset_carry(lane, pl, c);
 				for (uint32_t win = 0; win < n_win; ++win) {
 					phase_a<G, HALF_IN>(tid, win, A, sh.w, pl, st);
 					group_sync();
 					if (wave == 0) chain<G>(lane, win, A, sh.w, sh.rl, pl, c);
 					group_sync();
-					phase_c<G, HALF_IN, HALF_OUT>(tid, win, A, sh.w, sh.rl, pl, st);
-					group_sync();
 				}
+				if (wave == 0) finish_ray(lane, ray0, A, sh.rl, c, target, lo, hi);
+				if (!BACKWARD) {
+					if (live) S.side[ray0 + lane] = sh.rl.rnf[lane];
+				} else {
+					if (wave == 0) commit_ray(lane, ray0, live ? S.side[ray0 + lane] : 0u, A, sh.rl, pl, lo, hi);
+					group_sync();
+					if (wave == 0) reset_carry(lane, pl, c);
+					for (uint32_t win = 0; win < n_win; ++win) {
+						phase_a<G, HALF_IN>(tid, win, A, sh.w, pl, st);
+						group_sync();
+						if (wave == 0) chain<G>(lane, win, A, sh.w, sh.rl, pl, c);
+						group_sync();
+						phase_c<G, HALF_IN, HALF_OUT>(tid, win, A, sh.w, sh.rl, pl, st);
+						group_sync();
+					}
+				}
+				group_sync();
 			}
-		} else if (wave == 0) {
+		} else if (wave == 0 && slot == 0) {
+			const bool live = ray0 + lane < A.n_active;
 			uint32_t n = 0;
 			FwdRay fw;
 			loss_forward_body<HALF_IN>(ray0 + lane, A.K, A.rays_rgba, A.n_active, A.ray_coord_indices, A.dt_arr, A.net, &fw, &n, A.rgb_ray_out);
@@ -705,12 +761,13 @@ static int launch_stream(const srf_loss_args* a, const LossConst& K, ChainScratc
 #undef SRF_RESIDENT_IO
 #undef SRF_RESIDENT
 	if (rc != SRF_OK) return rc;
-	const dim3 grid(n_groups < resident ? n_groups : resident), block(STREAM_THREADS), slow_block(fused::WideGeometry::THREADS), slow_grid(n_groups < 256u ? n_groups : 256u);   // listed groups are few
+	const dim3 grid(n_groups < resident ? n_groups : resident), block(STREAM_THREADS), slow_block(fused::WideGeometry::THREADS), slow_grid(n_groups < SLOW_WORKGROUPS ? n_groups : SLOW_WORKGROUPS);   // listed groups are few as a rule
+	const uint32_t slow_slots = S.saved_records ? SLOW_PART_SLOTS : 1u;       // without the copy of their records a group is one workgroup's
 	hipLaunchKernelGGL(k_chain_prepare, dim3(div_up(n_groups, PREPARE_WAVES)), dim3(PREPARE_WAVES * WAVE), 0, st, A, n_rays_counter, S, (const uint32_t*)n_compacted_coords_counter);
 	hipLaunchKernelGGL(k_chain_items, dim3(div_up(n_groups, ITEMS_THREADS)), dim3(ITEMS_THREADS), 0, st, a->n_rays, n_rays_counter, S);
 	SRF_LAUNCH_CHECK();
-	if (hin) hipLaunchKernelGGL((k_slow_groups<true, false, false>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S);
-	else     hipLaunchKernelGGL((k_slow_groups<false, false, false>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S);
+	if (hin) hipLaunchKernelGGL((k_slow_groups<true, false, false>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S, slow_slots);
+	else     hipLaunchKernelGGL((k_slow_groups<false, false, false>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S, slow_slots);
 	SRF_LAUNCH_CHECK();
 #define SRF_STREAM(HI, HO, PL) hipLaunchKernelGGL((k_composite_stream<HI, HO, PL>), grid, block, 0, st, A, n_rays_counter, density_grid_mean, S, n_compacted_coords_counter)
 #define SRF_STREAM_IO(PL) do { if (hin && hout) SRF_STREAM(true, true, PL); else if (hin) SRF_STREAM(true, false, PL); else if (hout) SRF_STREAM(false, true, PL); else SRF_STREAM(false, false, PL); } while (0)
@@ -718,7 +775,7 @@ static int launch_stream(const srf_loss_args* a, const LossConst& K, ChainScratc
 #undef SRF_STREAM_IO
 #undef SRF_STREAM
 	SRF_LAUNCH_CHECK();
-#define SRF_SLOW_BWD(HI, HO) hipLaunchKernelGGL((k_slow_groups<HI, HO, true>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S)
+#define SRF_SLOW_BWD(HI, HO) hipLaunchKernelGGL((k_slow_groups<HI, HO, true>), slow_grid, slow_block, 0, st, A, n_rays_counter, density_grid_mean, S, slow_slots)
 	if (hin && hout) SRF_SLOW_BWD(true, true); else if (hin) SRF_SLOW_BWD(true, false); else if (hout) SRF_SLOW_BWD(false, true); else SRF_SLOW_BWD(false, false);
 #undef SRF_SLOW_BWD
 	SRF_LAUNCH_CHECK();
@@ -854,7 +911,7 @@ static int loss_call_prepare(srf_marcher* m, const srf_loss_args* a, const float
 // The chain's scratch for srf_marcher_volume_rendering_with_loss_and_gradient_noalloc: part of the library's image on every
 // device, found once per device with hipGetSymbolAddress (the array's name means nothing to host code).
 constexpr uint32_t NOALLOC_MAX_RAYS = SRF_NOALLOC_MAX_RAYS;
-constexpr size_t NOALLOC_BYTES = chain_layout(NOALLOC_MAX_RAYS, NOALLOC_MAX_PARTS).bytes;
+constexpr size_t NOALLOC_BYTES = chain_layout(NOALLOC_MAX_RAYS, NOALLOC_MAX_PARTS, false).bytes;
 static __device__ __align__(256) unsigned char g_noalloc_scratch[NOALLOC_BYTES];
 constexpr int NOALLOC_MAX_DEVICES = 64;
 static void* g_noalloc_ptr[NOALLOC_MAX_DEVICES];      // per device: where g_noalloc_scratch lies in its memory
@@ -973,10 +1030,10 @@ int srf_marcher_volume_rendering_with_loss_and_gradient(srf_marcher_t* m, const 
 		                    compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, st);
 	}
 	if (fusable && level == 0) {
-		rc = m->ws.reserve(chain_layout(a->n_rays, STREAM_MAX_PARTS).bytes);
+		rc = m->ws.reserve(chain_layout(a->n_rays, STREAM_MAX_PARTS, true).bytes);
 		if (rc != SRF_OK) return rc;
-		m->chain_error_dev = chain_scratch_at(m->ws.ptr, a->n_rays, STREAM_MAX_PARTS, nullptr, 0).error;
-		return launch_stream(a, K, chain_scratch_at(m->ws.ptr, a->n_rays, STREAM_MAX_PARTS, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
+		m->chain_error_dev = chain_scratch_at(m->ws.ptr, a->n_rays, STREAM_MAX_PARTS, true, nullptr, 0).error;
+		return launch_stream(a, K, chain_scratch_at(m->ws.ptr, a->n_rays, STREAM_MAX_PARTS, true, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
 		                     compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, st);
 	}
 
@@ -1033,8 +1090,8 @@ int srf_marcher_volume_rendering_with_loss_and_gradient_noalloc(srf_marcher_t* m
 	void* scratch = nullptr;
 	rc = noalloc_scratch(&scratch);
 	if (rc != SRF_OK) return rc;
-	m->chain_error_dev = chain_scratch_at(scratch, a->n_rays, NOALLOC_MAX_PARTS, nullptr, 0).error;
-	return launch_stream(a, K, chain_scratch_at(scratch, a->n_rays, NOALLOC_MAX_PARTS, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
+	m->chain_error_dev = chain_scratch_at(scratch, a->n_rays, NOALLOC_MAX_PARTS, false, nullptr, 0).error;
+	return launch_stream(a, K, chain_scratch_at(scratch, a->n_rays, NOALLOC_MAX_PARTS, false, m->host_error_dev, m->lookback_spin_limit), rays_rgba, n_rays_counter, ray_coord_indices, dt, coords,
 	                     compacted_coords, n_compacted_coords_counter, network_output, dloss_doutput, loss_output, density_grid_mean, rgb_ray_out, (hipStream_t)stream);
 }
 

@@ -120,6 +120,23 @@ SRF_HD uint64_t plan_cuts(const Plan& pl, uint32_t max_parts) {
 	return cuts;
 }
 
+// Where the kernel for the listed groups cuts a group whose rays lie back to back: as plan_cuts, except that a ray longer than
+// a window is a part of its own (that kernel takes a part through as many windows as it needs).
+template <class G>
+SRF_HD uint64_t plan_cuts_any_length(const Plan& pl) {
+	const uint32_t total = pl.misc[M_TOTAL];
+	uint64_t cuts = 1ull;
+	uint32_t lo = 0;
+	for (;;) {
+		uint32_t r = lo;      // the first ray from lo on that ends beyond the window beginning with ray lo
+		while (r < RAYS && (r + 1 < RAYS ? pl.rbase[r + 1] : total) - pl.rbase[lo] <= G::WIN) ++r;
+		if (r == lo) ++r;     // ray lo alone is longer than a window
+		if (r >= RAYS) return cuts;
+		lo = r;
+		cuts |= 1ull << lo;
+	}
+}
+
 // The plan of rays [lo, hi) of a planned group, one lane per ray: the other rays own nothing in it.
 SRF_HD void plan_part_lane(uint32_t lane, const Plan& group, uint32_t lo, uint32_t hi, uint32_t g, Plan& part) {
 	const uint32_t start = group.rbase[lo];
@@ -252,9 +269,9 @@ SRF_HD void plan_lane(uint32_t lane, uint32_t ray0, const Args& A, Plan& pl) {
 	}
 	if (lane == 0) {
 		const uint64_t end = n_here ? (uint64_t)pl.rabs[n_here - 1] + pl.rn[n_here - 1] : 0;
-		const uint64_t total = end >= s0 ? end - s0 : 0;
 		pl.misc[M_S0] = s0;
-		pl.misc[M_TOTAL] = total > 0xffffffffull ? 0xffffffffu : (uint32_t)total;
+		pl.misc[M_TOTAL] = (uint32_t)end - s0;      // modulo 2^32: in the plan of a part of the group the first ray's offset cancels
+		if (!(end >= s0 && end - s0 <= 0xffffffffull)) SRF_LDS_AND(&pl.misc[M_CONTIG], 0u);
 	}
 }
 

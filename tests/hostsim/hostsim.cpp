@@ -115,22 +115,32 @@ static void run_fused(const orc_loss_args* a, const float* rays_rgba, uint32_t n
 			std::vector<Float4> tgt(RAYS);
 			make_plan(g, pl, &tgt);
 			if (pl.misc[M_CONTIG] != 0) {
-				const uint32_t n_win = (pl.misc[M_TOTAL] + GW::WIN - 1) / GW::WIN;
-				for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
-				for (uint32_t win = 0; win < n_win; ++win) {
-					for (uint32_t t = 0; t < GW::THREADS; ++t) phase_a<GW, HI>(t, win, B, *ww, pl, st_w[t]);
-					for (uint32_t t = 0; t < RAYS; ++t) chain<GW>(t, win, B, *ww, rl, pl, c[t]);
-				}
-				for (uint32_t t = 0; t < RAYS; ++t) finish_ray(t, ray0, B, rl, c[t], tgt[t]);
-				if (!backward) {
-					for (uint32_t t = 0; t < RAYS; ++t) if (ray0 + t < B.n_active) side[ray0 + t] = rl.rnf[t];
-				} else {
-					for (uint32_t t = 0; t < RAYS; ++t) commit_ray(t, ray0, ray0 + t < B.n_active ? side[ray0 + t] : 0u, B, rl, pl);
+				// part by part (the device deals a group's parts to several workgroups)
+				Plan group = pl;
+				uint64_t cuts = plan_cuts_any_length<GW>(group);
+				while (cuts) {
+					const uint32_t lo = (uint32_t)__builtin_ctzll(cuts);
+					cuts &= cuts - 1ull;
+					const uint32_t hi = cuts ? (uint32_t)__builtin_ctzll(cuts) : RAYS;
+					for (uint32_t t = 0; t < RAYS; ++t) plan_part_lane(t, group, lo, hi, g, pl);
+					const uint32_t n_win = (pl.misc[M_TOTAL] + GW::WIN - 1) / GW::WIN;
+					auto live = [&](uint32_t t) { return ray0 + t < B.n_active && t >= lo && t < hi; };
 					for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
 					for (uint32_t win = 0; win < n_win; ++win) {
 						for (uint32_t t = 0; t < GW::THREADS; ++t) phase_a<GW, HI>(t, win, B, *ww, pl, st_w[t]);
 						for (uint32_t t = 0; t < RAYS; ++t) chain<GW>(t, win, B, *ww, rl, pl, c[t]);
-						for (uint32_t t = 0; t < GW::THREADS; ++t) phase_c<GW, HI, HO>(t, win, B, *ww, rl, pl, st_w[t]);
+					}
+					for (uint32_t t = 0; t < RAYS; ++t) finish_ray(t, ray0, B, rl, c[t], tgt[t], lo, hi);
+					if (!backward) {
+						for (uint32_t t = 0; t < RAYS; ++t) if (live(t)) side[ray0 + t] = rl.rnf[t];
+					} else {
+						for (uint32_t t = 0; t < RAYS; ++t) commit_ray(t, ray0, live(t) ? side[ray0 + t] : 0u, B, rl, pl, lo, hi);
+						for (uint32_t t = 0; t < RAYS; ++t) reset_carry(t, pl, c[t]);
+						for (uint32_t win = 0; win < n_win; ++win) {
+							for (uint32_t t = 0; t < GW::THREADS; ++t) phase_a<GW, HI>(t, win, B, *ww, pl, st_w[t]);
+							for (uint32_t t = 0; t < RAYS; ++t) chain<GW>(t, win, B, *ww, rl, pl, c[t]);
+							for (uint32_t t = 0; t < GW::THREADS; ++t) phase_c<GW, HI, HO>(t, win, B, *ww, rl, pl, st_w[t]);
+						}
 					}
 				}
 			} else {
