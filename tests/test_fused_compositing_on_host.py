@@ -151,3 +151,41 @@ def test_fused_handles_empty_and_inactive_batches(orc, hostsim):
         for other in res[1:]:
             for x, y in zip(res[0], other):
                 assert np.array_equal(x, y)
+
+
+@pytest.mark.parametrize("kind", ["split", "parts"])
+def test_items_of_a_cut_group_do_not_depend_on_records_already_overwritten(orc, hostsim, kind):
+    """The commit writes a ray's compacted count and offset over its record.  An item of a cut group is planned after
+    the items before it have committed (always in this host build, now and then on the device), so its plan must come out
+    of its own rays' records whatever the earlier rays' now hold: here offsets far above every sample index, because the
+    compacted counter starts there."""
+    rng = np.random.default_rng(5)
+    n_rays = 64 * 3 + 11
+    counts, base, total = layout(rng, kind, n_rays)
+    net = helpers.random_network_output(rng, total)
+    net[:, 3] *= 0.05
+    dt = (rng.random(total) * 0.3 + 0.01).astype(np.float32)
+    tgt = rng.random((n_rays, 4)).astype(np.float32)
+    start = 0xF0000000
+    cap = start      # no room behind the counter's starting value: every ray keeps nothing, so no gradient is written up there
+    a = loss_args(n_rays, cap)
+    res = []
+    for fn in ("oracle", "fused"):
+        idx = np.stack([counts, base], axis=1).astype(np.uint32)
+        dloss = np.zeros((16, 4), np.float32)
+        loss = np.full(n_rays, -1, np.float32)
+        rgb = np.zeros((n_rays, 3), np.float32)
+        if fn == "oracle":
+            tot = orc.volume_rendering_with_loss_and_gradient(a, tgt, n_rays, idx, dt, net, dloss, n_compacted_counter=start, loss_output=loss, rgb_ray_out=rgb)
+        else:
+            cnt = np.array([start], np.uint32)
+            ns, nm = C.c_uint32(), C.c_uint32()
+            hostsim.lib.hs_loss_fused(C.byref(a), ptr(tgt), n_rays, ptr(idx), ptr(dt), None, None, ptr(cnt), ptr(net), ptr(dloss), ptr(loss), ptr(rgb),
+                                      C.byref(ns), C.byref(nm))
+            tot = int(cnt[0])
+            assert ns.value == 0 and nm.value == 0
+        assert not dloss.any()
+        res.append((tot, idx, loss, rgb))
+    for x, y in zip(res[0], res[1]):
+        assert np.array_equal(x, y)
+    assert res[0][0] > start and res[0][3].any()
