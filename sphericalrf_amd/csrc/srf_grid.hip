@@ -138,19 +138,27 @@ __global__ void __launch_bounds__(256) k_grid_samples_to_point_order(uint32_t n_
 // summary_a (cleared by the caller): bit (w & 31) of word (w >> 5) is set where word w of above_a has a bit that is not set
 __global__ void __launch_bounds__(256) k_threshold_bits(const float* __restrict__ grid, uint32_t n_total, float thresh_a, float thresh_b,
                                                          uint32_t* __restrict__ above_a, uint32_t* __restrict__ above_b, uint32_t* __restrict__ summary_a) {
+	constexpr uint32_t ROUNDS = 4;      // 64-cell rounds a wavefront has in flight: four independent loads a lane
 	const uint32_t lane = threadIdx.x & 63u;
-	const uint32_t stride = gridDim.x * blockDim.x;
-	for (uint32_t base = (blockIdx.x * blockDim.x + threadIdx.x) - lane; base < n_total; base += stride) {   // uniform per wavefront
-		const uint32_t i = base + lane;
-		const float v = i < n_total ? grid[i] : 0.f;
-		const uint64_t ma = __ballot(i < n_total && v > thresh_a), mb = __ballot(i < n_total && v > thresh_b);
-		if (lane == 0) {
-			above_a[base >> 5] = (uint32_t)ma; above_b[base >> 5] = (uint32_t)mb;
-			const uint32_t w = base >> 5;      // (even: both words of the round share a summary word)
-			const uint32_t some = ((uint32_t)ma != 0xffffffffu ? 1u : 0u) | ((uint32_t)(ma >> 32) != 0xffffffffu ? 2u : 0u);
-			if (some) atomicOr(&summary_a[w >> 5], some << (w & 31u));
+	const uint32_t stride = gridDim.x * blockDim.x * ROUNDS;
+	for (uint32_t first = ((blockIdx.x * blockDim.x + threadIdx.x) - lane) * ROUNDS; first < n_total; first += stride) {   // uniform per wavefront
+		float v[ROUNDS];
+		#pragma unroll
+		for (uint32_t k = 0; k < ROUNDS; ++k) { const uint32_t i = first + k * 64u + lane; v[k] = i < n_total ? grid[i] : 0.f; }
+		#pragma unroll
+		for (uint32_t k = 0; k < ROUNDS; ++k) {
+			const uint32_t base = first + k * 64u;
+			if (base >= n_total) break;
+			const uint32_t i = base + lane;
+			const uint64_t ma = __ballot(i < n_total && v[k] > thresh_a), mb = __ballot(i < n_total && v[k] > thresh_b);
+			if (lane == 0) {
+				above_a[base >> 5] = (uint32_t)ma; above_b[base >> 5] = (uint32_t)mb;
+				const uint32_t w = base >> 5;      // (even: both words of the round share a summary word)
+				const uint32_t some = ((uint32_t)ma != 0xffffffffu ? 1u : 0u) | ((uint32_t)(ma >> 32) != 0xffffffffu ? 2u : 0u);
+				if (some) atomicOr(&summary_a[w >> 5], some << (w & 31u));
+			}
+			if (lane == 32 && base + 32 < n_total) { above_a[(base >> 5) + 1] = (uint32_t)(ma >> 32); above_b[(base >> 5) + 1] = (uint32_t)(mb >> 32); }
 		}
-		if (lane == 32 && base + 32 < n_total) { above_a[(base >> 5) + 1] = (uint32_t)(ma >> 32); above_b[(base >> 5) + 1] = (uint32_t)(mb >> 32); }
 	}
 }
 
@@ -885,7 +893,7 @@ int srf_sampler_sample_positions_from_grid(srf_sampler_t* s, uint32_t n_uniform,
 		uint32_t* sum = (uint32_t*)((char*)s->ws.ptr + 2 * table_bytes);
 		rc = fill_u32(sum, summary_words, 0u, st);
 		if (rc != SRF_OK) return rc;
-		const uint32_t blocks = div_up(s->n_total, 256) < 16384 ? div_up(s->n_total, 256) : 16384;
+		const uint32_t blocks = div_up(s->n_total, 1024) < 16384 ? div_up(s->n_total, 1024) : 16384;
 		hipLaunchKernelGGL(k_threshold_bits, dim3(blocks), dim3(256), 0, st, (const float*)s->density_grid, s->n_total, -0.01f, s->P.min_optical_thickness, a, b, sum);
 		SRF_LAUNCH_CHECK();
 		above_a = a; above_b = b; summary_a = sum;
